@@ -1,0 +1,223 @@
+// C ABI: handle lifecycle, argument validation and dispatch to the kernel families.
+// Validation happens entirely on the host, before any launch: a call that returns a
+// non-success status has enqueued nothing.
+#include <cstdarg>
+#include <cstdlib>
+#include <new>
+
+#include "common.h"
+
+namespace cig {
+
+cigemmStatus_t fail(cigemmContext* ctx, cigemmStatus_t st, const char* fmt, ...) {
+  if (ctx) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(ctx->last_error, sizeof(ctx->last_error), fmt, ap);
+    va_end(ap);
+  }
+  return st;
+}
+
+cigemmStatus_t check_launch(cigemmContext* ctx, const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(ctx, CIGEMM_STATUS_EXECUTION_FAILED, "%s: HIP error: %s", what,
+                hipGetErrorString(e));
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+namespace {
+
+bool valid(cigemmHandle_t h) { return h && h->magic == kCtxMagic; }
+
+// Common checks of one C[MxN] = A[MxK] . B GEMM call.  b_rows x b_cols is B's stored shape.
+cigemmStatus_t check_gemm_args(cigemmHandle_t h, const char* name, int64_t M, int64_t N,
+                               int64_t K, const void* A, int64_t lda, const void* B,
+                               int64_t ldb, int64_t b_cols, const void* C, int64_t ldc) {
+  if (M < 0 || N < 0 || K < 0)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: negative dimension (M=%lld N=%lld K=%lld)",
+                name, (long long)M, (long long)N, (long long)K);
+  if (M == 0 || N == 0) return CIGEMM_STATUS_SUCCESS;
+  if (!C) return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: null output pointer", name);
+  if (ldc < N)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: ldc=%lld < N=%lld", name, (long long)ldc,
+                (long long)N);
+  if (K > 0) {
+    if (!A || !B) return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: null input pointer", name);
+    if (lda < K)
+      return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: lda=%lld < K=%lld", name, (long long)lda,
+                  (long long)K);
+    if (ldb < b_cols)
+      return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: ldb=%lld < %lld", name, (long long)ldb,
+                  (long long)b_cols);
+  }
+  if ((M + 63) / 64 > 65535)
+    return fail(h, CIGEMM_STATUS_NOT_SUPPORTED, "%s: M=%lld exceeds the launch grid", name,
+                (long long)M);
+  if (K > 2147483647LL || N > 2147483647LL)
+    return fail(h, CIGEMM_STATUS_NOT_SUPPORTED, "%s: N or K exceeds 2^31-1", name);
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+}  // namespace
+}  // namespace cig
+
+using namespace cig;
+
+extern "C" {
+
+cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
+  if (!handle) return CIGEMM_STATUS_INVALID_VALUE;
+  *handle = nullptr;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return CIGEMM_STATUS_NOT_INITIALIZED;
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return CIGEMM_STATUS_NOT_INITIALIZED;
+  }
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return CIGEMM_STATUS_ARCH_MISMATCH;
+  cigemmContext* ctx = new (std::nothrow) cigemmContext();
+  if (!ctx) return CIGEMM_STATUS_ALLOC_FAILED;
+  ctx->magic = kCtxMagic;
+  ctx->device = dev;
+  ctx->num_cus = prop.multiProcessorCount;
+  ctx->stream = nullptr;
+  ctx->last_kernel = "";
+  ctx->last_error[0] = '\0';
+  *handle = ctx;
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+cigemmStatus_t cigemmDestroy(cigemmHandle_t h) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  h->magic = 0;
+  delete h;
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+cigemmStatus_t cigemmSetStream(cigemmHandle_t h, void* stream) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  h->stream = static_cast<hipStream_t>(stream);
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+cigemmStatus_t cigemmGetStream(cigemmHandle_t h, void** stream) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if (!stream) return fail(h, CIGEMM_STATUS_INVALID_VALUE, "cigemmGetStream: null argument");
+  *stream = h->stream;
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+const char* cigemmGetStatusString(cigemmStatus_t status) {
+  switch (status) {
+    case CIGEMM_STATUS_SUCCESS: return "CIGEMM_STATUS_SUCCESS";
+    case CIGEMM_STATUS_NOT_INITIALIZED: return "CIGEMM_STATUS_NOT_INITIALIZED";
+    case CIGEMM_STATUS_ALLOC_FAILED: return "CIGEMM_STATUS_ALLOC_FAILED";
+    case CIGEMM_STATUS_INVALID_VALUE: return "CIGEMM_STATUS_INVALID_VALUE";
+    case CIGEMM_STATUS_ARCH_MISMATCH: return "CIGEMM_STATUS_ARCH_MISMATCH";
+    case CIGEMM_STATUS_EXECUTION_FAILED: return "CIGEMM_STATUS_EXECUTION_FAILED";
+    case CIGEMM_STATUS_INTERNAL_ERROR: return "CIGEMM_STATUS_INTERNAL_ERROR";
+    case CIGEMM_STATUS_NOT_SUPPORTED: return "CIGEMM_STATUS_NOT_SUPPORTED";
+    default: return "CIGEMM_STATUS_UNKNOWN";
+  }
+}
+
+const char* cigemmGetLastErrorString(cigemmHandle_t h) { return valid(h) ? h->last_error : ""; }
+
+int cigemmGetVersion(void) { return 100; }
+
+const char* cigemmGetLastKernelName(cigemmHandle_t h) { return valid(h) ? h->last_kernel : ""; }
+
+cigemmStatus_t cigemm_gemm_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K, const float* A,
+                               int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  cigemmStatus_t st = check_gemm_args(h, "cigemm_gemm_f32", M, N, K, A, lda, B, ldb, N, C, ldc);
+  if (st != CIGEMM_STATUS_SUCCESS || M == 0 || N == 0) return st;
+  if (!launch_f32_mfma(h, M, N, K, A, lda, B, ldb, C, ldc))
+    launch_generic_f32(h, M, N, K, A, lda, B, ldb, C, ldc);
+  return check_launch(h, "cigemm_gemm_f32");
+}
+
+static cigemmStatus_t gemm16(cigemmHandle_t h, const char* name, bool bf16, int64_t M, int64_t N,
+                             int64_t K, const uint16_t* A, int64_t lda, const uint16_t* B,
+                             int64_t ldb, uint16_t* C, int64_t ldc) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  cigemmStatus_t st = check_gemm_args(h, name, M, N, K, A, lda, B, ldb, N, C, ldc);
+  if (st != CIGEMM_STATUS_SUCCESS || M == 0 || N == 0) return st;
+  if (!launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc) &&
+      !launch_skinny_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc))
+    launch_generic_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc);
+  return check_launch(h, name);
+}
+
+cigemmStatus_t cigemm_gemm_f16(cigemmHandle_t h, int64_t M, int64_t N, int64_t K,
+                               const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
+                               uint16_t* C, int64_t ldc) {
+  return gemm16(h, "cigemm_gemm_f16", false, M, N, K, A, lda, B, ldb, C, ldc);
+}
+
+cigemmStatus_t cigemm_gemm_bf16(cigemmHandle_t h, int64_t M, int64_t N, int64_t K,
+                                const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
+                                uint16_t* C, int64_t ldc) {
+  return gemm16(h, "cigemm_gemm_bf16", true, M, N, K, A, lda, B, ldb, C, ldc);
+}
+
+static cigemmStatus_t gemm_i8(cigemmHandle_t h, const char* name, int64_t M, int64_t N, int64_t K,
+                              const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb,
+                              cigemmBLayout_t b_layout, int32_t* C, int64_t ldc,
+                              const DequantArgs* dq) {
+  const bool b_nk = b_layout == CIGEMM_B_NK;
+  if (!launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq) &&
+      !launch_skinny_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq))
+    launch_generic_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);
+  return check_launch(h, name);
+}
+
+cigemmStatus_t cigemm_gemm_i8_i32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K,
+                                  const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb,
+                                  cigemmBLayout_t b_layout, int32_t* C, int64_t ldc) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if (b_layout != CIGEMM_B_KN && b_layout != CIGEMM_B_NK)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "cigemm_gemm_i8_i32: bad b_layout %d",
+                (int)b_layout);
+  cigemmStatus_t st = check_gemm_args(h, "cigemm_gemm_i8_i32", M, N, K, A, lda, B, ldb,
+                                      b_layout == CIGEMM_B_NK ? K : N, C, ldc);
+  if (st != CIGEMM_STATUS_SUCCESS || M == 0 || N == 0) return st;
+  return gemm_i8(h, "cigemm_gemm_i8_i32", M, N, K, A, lda, B, ldb, b_layout, C, ldc, nullptr);
+}
+
+cigemmStatus_t cigemm_gemm_i8_dequant(cigemmHandle_t h, int64_t M, int64_t N, int64_t K,
+                                      const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb,
+                                      cigemmBLayout_t b_layout, const float* scaleA,
+                                      cigemmScaleMode_t scaleA_mode, const float* scaleB,
+                                      cigemmScaleMode_t scaleB_mode, void* out,
+                                      cigemmOutType_t out_type, int64_t ldo, int32_t* acc_out,
+                                      int64_t ldacc) {
+  const char* name = "cigemm_gemm_i8_dequant";
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if (b_layout != CIGEMM_B_KN && b_layout != CIGEMM_B_NK)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: bad b_layout %d", name, (int)b_layout);
+  if ((scaleA_mode != CIGEMM_SCALE_TENSOR && scaleA_mode != CIGEMM_SCALE_VECTOR) ||
+      (scaleB_mode != CIGEMM_SCALE_TENSOR && scaleB_mode != CIGEMM_SCALE_VECTOR))
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: bad scale mode", name);
+  if (out_type != CIGEMM_OUT_F32 && out_type != CIGEMM_OUT_BF16)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: bad out_type %d", name, (int)out_type);
+  cigemmStatus_t st = check_gemm_args(h, name, M, N, K, A, lda, B, ldb,
+                                      b_layout == CIGEMM_B_NK ? K : N, out, ldo);
+  if (st != CIGEMM_STATUS_SUCCESS || M == 0 || N == 0) return st;
+  if (!scaleA || !scaleB) return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: null scale pointer", name);
+  if (acc_out && ldacc < N)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: ldacc=%lld < N=%lld", name, (long long)ldacc,
+                (long long)N);
+  DequantArgs dq{scaleA, scaleB, scaleA_mode == CIGEMM_SCALE_VECTOR,
+                 scaleB_mode == CIGEMM_SCALE_VECTOR, out, out_type == CIGEMM_OUT_BF16, ldo,
+                 acc_out, ldacc};
+  return gemm_i8(h, name, M, N, K, A, lda, B, ldb, b_layout, nullptr, 0, &dq);
+}
+
+}  // extern "C"

@@ -1,0 +1,172 @@
+// Shared declarations of the gfx950 GEMM library: context, status plumbing, vector types,
+// narrowing conversions and the epilogue functors every kernel family uses.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "cigemm.h"
+
+struct cigemmContext {
+  uint32_t magic;
+  int device;
+  int num_cus;
+  hipStream_t stream;
+  const char* last_kernel;
+  char last_error[256];
+};
+
+constexpr uint32_t kCtxMagic = 0xC16E3350u;
+
+namespace cig {
+
+// ---- status plumbing ------------------------------------------------------------------
+cigemmStatus_t fail(cigemmContext* ctx, cigemmStatus_t st, const char* fmt, ...)
+    __attribute__((format(printf, 3, 4)));
+cigemmStatus_t check_launch(cigemmContext* ctx, const char* what);
+
+// ---- vector types ---------------------------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// ---- element conversions (device) -----------------------------------------------------
+// bfloat16: round to nearest even on the bit pattern; NaN keeps its sign and is quieted.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
+  return __builtin_bit_cast(float, (uint32_t)h << 16);
+}
+// binary16: the hardware conversion rounds to nearest even in the default FP mode.
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;
+  return __builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+
+// Element tags: how a 16-bit pattern is widened / narrowed.
+struct BF16 {
+  static __device__ __forceinline__ float widen(uint16_t h) { return bf16_bits_to_f32(h); }
+  static __device__ __forceinline__ uint16_t narrow(float f) { return f32_to_bf16_bits(f); }
+};
+struct F16 {
+  static __device__ __forceinline__ float widen(uint16_t h) { return f16_bits_to_f32(h); }
+  static __device__ __forceinline__ uint16_t narrow(float f) { return f32_to_f16_bits(f); }
+};
+
+// ---- epilogues --------------------------------------------------------------------------
+// Each epilogue stores one accumulator for output element (row, col).
+
+struct EpiStoreF32 {  // fp32 GEMM
+  float* C;
+  int64_t ldc;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float acc) const {
+    C[r * ldc + c] = acc;
+  }
+};
+
+template <typename E16>
+struct EpiStore16 {  // fp16 / bf16 GEMM: one narrowing of the fp32 accumulator
+  uint16_t* C;
+  int64_t ldc;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float acc) const {
+    C[r * ldc + c] = E16::narrow(acc);
+  }
+};
+
+struct EpiStoreI32 {  // int8 GEMM, raw accumulators
+  int32_t* C;
+  int64_t ldc;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, int32_t acc) const {
+    C[r * ldc + c] = acc;
+  }
+};
+
+// out = ((float)acc * sA) * sB, two separately rounded fp32 multiplies.  The float
+// conversion of the accumulator rounds to nearest even (v_cvt_f32_i32).
+template <bool OUT_BF16, bool DUMP_ACC>
+struct EpiDequant {
+  void* out;
+  int64_t ldo;
+  const float* sa;
+  const float* sb;
+  int sa_vec;  // 1: sa[row], 0: sa[0]
+  int sb_vec;  // 1: sb[col], 0: sb[0]
+  int32_t* acc_out;
+  int64_t ldacc;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, int32_t acc) const {
+    const float a = sa[sa_vec ? r : 0];
+    const float b = sb[sb_vec ? c : 0];
+    const float v = __fmul_rn(__fmul_rn((float)acc, a), b);
+    if (OUT_BF16)
+      static_cast<uint16_t*>(out)[r * ldo + c] = f32_to_bf16_bits(v);
+    else
+      static_cast<float*>(out)[r * ldo + c] = v;
+    if (DUMP_ACC) acc_out[r * ldacc + c] = acc;
+  }
+};
+
+struct DequantArgs {
+  const float* sa;
+  const float* sb;
+  int sa_vec;
+  int sb_vec;
+  void* out;
+  int out_bf16;
+  int64_t ldo;
+  int32_t* acc_out;
+  int64_t ldacc;
+};
+
+// ---- kernel-family entry points (host side, defined in the per-family .hip files) ------
+// Each returns true when it took the problem (launched), false when the shape or the
+// alignment is outside what that family handles; the caller then falls through to the
+// generic kernel.
+
+// gemm_generic.hip: any shape, any alignment.
+void launch_generic_f32(cigemmContext*, int64_t M, int64_t N, int64_t K, const float* A,
+                        int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc);
+void launch_generic_16(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
+                       const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
+                       uint16_t* C, int64_t ldc);
+void launch_generic_i8(cigemmContext*, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                       int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
+                       int64_t ldc, const DequantArgs* dq);
+
+// gemm_f32.hip
+bool launch_f32_mfma(cigemmContext*, int64_t M, int64_t N, int64_t K, const float* A,
+                     int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc);
+// gemm_16b.hip
+bool launch_16b_mfma(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
+                     const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
+                     uint16_t* C, int64_t ldc);
+// gemm_i8.hip
+bool launch_i8_mfma(cigemmContext*, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                    int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
+                    int64_t ldc, const DequantArgs* dq);
+// gemm_skinny.hip
+bool launch_skinny_16(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
+                      const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
+                      uint16_t* C, int64_t ldc);
+bool launch_skinny_i8(cigemmContext*, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                      int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
+                      int64_t ldc, const DequantArgs* dq);
+
+}  // namespace cig

@@ -1,0 +1,43 @@
+// fp16 / bf16 GEMM on the gfx950 matrix cores: C[MxN] = A[MxK] . B[KxN], row-major, 16-bit
+// in, fp32 accumulate (v_mfma_f32_32x32x16_{f16,bf16}), one round-to-nearest-even narrowing
+// out.  The kernel itself is the shared LDS-tiled MFMA kernel; this file supplies the
+// 16-bit epilogue and the shape gate.
+#include "mfma_tile.h"
+
+namespace cig {
+namespace {
+
+// Narrows four consecutive columns and stores them as one 8-byte piece.
+template <typename E16>
+struct EpiStore16x4 {
+  uint16_t* C;
+  int64_t ldc;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float v0, float v1, float v2,
+                                             float v3) const {
+    u32x2 v;
+    v[0] = (uint32_t)E16::narrow(v0) | ((uint32_t)E16::narrow(v1) << 16);
+    v[1] = (uint32_t)E16::narrow(v2) | ((uint32_t)E16::narrow(v3) << 16);
+    *reinterpret_cast<u32x2*>(C + r * ldc + c) = v;
+  }
+};
+
+}  // namespace
+
+bool launch_16b_mfma(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_t K,
+                     const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, uint16_t* C,
+                     int64_t ldc) {
+  if (!tile::tile_shape_ok(M, N, K, 2, A, lda, B, ldb)) return false;
+  if (ldc % 4 || ((uintptr_t)C & 7)) return false;
+  if (bf16) {
+    tile::launch_tile<tile::MathBF16, tile::B_KN16>(ctx, M, N, K * 2, A, lda * 2, B, ldb * 2,
+                                                    EpiStore16x4<BF16>{C, ldc});
+    ctx->last_kernel = "bf16_mfma_256x256x64";
+  } else {
+    tile::launch_tile<tile::MathF16, tile::B_KN16>(ctx, M, N, K * 2, A, lda * 2, B, ldb * 2,
+                                                   EpiStore16x4<F16>{C, ldc});
+    ctx->last_kernel = "f16_mfma_256x256x64";
+  }
+  return true;
+}
+
+}  // namespace cig

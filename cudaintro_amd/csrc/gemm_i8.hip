@@ -1,0 +1,105 @@
+// int8 GEMM on the gfx950 matrix cores (v_mfma_i32_32x32x32_i8, exact int32 accumulation)
+// with either raw int32 output or the fused scale-and-dequantize epilogue.  The kernel is
+// the shared LDS-tiled MFMA kernel; this file supplies the int8 epilogues and the gate.
+#include "mfma_tile.h"
+
+namespace cig {
+namespace {
+
+struct EpiStoreI32x4 {
+  int32_t* C;
+  int64_t ldc;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, int32_t v0, int32_t v1,
+                                             int32_t v2, int32_t v3) const {
+    i32x4 v = {v0, v1, v2, v3};
+    *reinterpret_cast<i32x4*>(C + r * ldc + c) = v;
+  }
+};
+
+// out = ((float)acc * sA[row]) * sB[col]: two separately rounded fp32 multiplies, then an
+// optional round-to-nearest-even narrowing to bf16.  Four consecutive columns per call.
+template <bool OUT_BF16, bool DUMP_ACC>
+struct EpiDequantX4 {
+  void* out;
+  int64_t ldo;
+  const float* sa;
+  const float* sb;
+  int sa_vec, sb_vec;
+  int32_t* acc_out;
+  int64_t ldacc;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, int32_t v0, int32_t v1,
+                                             int32_t v2, int32_t v3) const {
+    const float a = sa[sa_vec ? r : 0];
+    f32x4 b;
+    if (sb_vec)
+      b = *reinterpret_cast<const f32x4*>(sb + c);
+    else
+      b = f32x4{sb[0], sb[0], sb[0], sb[0]};
+    float o[4];
+    o[0] = __fmul_rn(__fmul_rn((float)v0, a), b[0]);
+    o[1] = __fmul_rn(__fmul_rn((float)v1, a), b[1]);
+    o[2] = __fmul_rn(__fmul_rn((float)v2, a), b[2]);
+    o[3] = __fmul_rn(__fmul_rn((float)v3, a), b[3]);
+    if (OUT_BF16) {
+      u32x2 p;
+      p[0] = (uint32_t)f32_to_bf16_bits(o[0]) | ((uint32_t)f32_to_bf16_bits(o[1]) << 16);
+      p[1] = (uint32_t)f32_to_bf16_bits(o[2]) | ((uint32_t)f32_to_bf16_bits(o[3]) << 16);
+      *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + r * ldo + c) = p;
+    } else {
+      *reinterpret_cast<f32x4*>(static_cast<float*>(out) + r * ldo + c) =
+          f32x4{o[0], o[1], o[2], o[3]};
+    }
+    if (DUMP_ACC) {
+      i32x4 v = {v0, v1, v2, v3};
+      *reinterpret_cast<i32x4*>(acc_out + r * ldacc + c) = v;
+    }
+  }
+};
+
+template <int BMODE>
+void launch_layout(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                   int64_t lda, const int8_t* B, int64_t ldb, int32_t* C, int64_t ldc,
+                   const DequantArgs* dq) {
+  if (!dq) {
+    tile::launch_tile<tile::MathI8, BMODE>(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32x4{C, ldc});
+    return;
+  }
+#define CIG_DQ(OB, DA)                                                                        \
+  tile::launch_tile<tile::MathI8, BMODE>(                                                     \
+      ctx, M, N, K, A, lda, B, ldb,                                                           \
+      EpiDequantX4<OB, DA>{dq->out, dq->ldo, dq->sa, dq->sb, dq->sa_vec, dq->sb_vec,          \
+                           dq->acc_out, dq->ldacc})
+  const bool dump = dq->acc_out != nullptr;
+  if (dq->out_bf16) {
+    if (dump) CIG_DQ(true, true); else CIG_DQ(true, false);
+  } else {
+    if (dump) CIG_DQ(false, true); else CIG_DQ(false, false);
+  }
+#undef CIG_DQ
+}
+
+}  // namespace
+
+bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                    int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C, int64_t ldc,
+                    const DequantArgs* dq) {
+  if (!tile::tile_shape_ok(M, N, K, 1, A, lda, B, ldb)) return false;
+  if (!dq) {
+    if (ldc % 4 || ((uintptr_t)C & 15)) return false;
+  } else {
+    if (dq->out_bf16 ? (dq->ldo % 4 || ((uintptr_t)dq->out & 7))
+                     : (dq->ldo % 4 || ((uintptr_t)dq->out & 15)))
+      return false;
+    if (dq->sb_vec && ((uintptr_t)dq->sb & 15)) return false;
+    if (dq->acc_out && (dq->ldacc % 4 || ((uintptr_t)dq->acc_out & 15))) return false;
+  }
+  if (b_nk)
+    launch_layout<tile::B_NK>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
+  else
+    launch_layout<tile::B_KN8>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
+  ctx->last_kernel = dq ? (b_nk ? "i8_mfma_256x256x128_nk_dequant" : "i8_mfma_256x256x128_kn_dequant")
+                        : (b_nk ? "i8_mfma_256x256x128_nk" : "i8_mfma_256x256x128_kn");
+  return true;
+}
+
+}  // namespace cig

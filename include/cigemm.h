@@ -1,0 +1,172 @@
+/*
+ * cigemm.h -- C ABI of the MI355X (gfx950) quantization-GEMM library.
+ *
+ * This is the operator-level boundary: what the reference's quantization/ suite reaches
+ * through cuBLAS (cublasCreate / cublasSetMathMode / cublasGemmEx / cublasDestroy:
+ * quantization/main.cu:10-11,29 and the cublasGemmEx call sites in
+ * quantization/GEMM_{fp32,bf16,fp16,int8}.cu) plus its four device fill kernels.
+ * Reference paths below are relative to the reference repository root.
+ *
+ * Conventions
+ *   - Plain C: pointers, sizes, status codes.  No C++ or framework types.
+ *   - All matrices are ROW-MAJOR with explicit leading dimensions counted in elements
+ *     (the reference's CPU GEMM, TileProgramming/tensor_utils.cu:34-45, is row-major).
+ *   - C = A . B only (alpha = 1, beta = 0: all the reference ever passes,
+ *     quantization/GEMM_bf16.cu:48-49, GEMM_int8.cu:48-49).
+ *   - Every matrix pointer is DEVICE memory; calls enqueue on the handle's stream and
+ *     return without synchronising (like cublasGemmEx).  Nothing is allocated per call.
+ *   - Errors come back as codes; the library never exits the process.  The message of
+ *     the last failing call on a handle is kept in cigemmGetLastErrorString().
+ *   - A handle is not thread-safe; use one per host thread.
+ *   - There is no CPU fallback: without a gfx950 device cigemmCreate() fails.
+ */
+#ifndef CIGEMM_H_
+#define CIGEMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CIGEMM_API __attribute__((visibility("default")))
+
+/* Mirrors the cublasStatus_t values the reference prints
+ * (quantization/gemm_common.h:10-35). */
+typedef enum cigemmStatus {
+  CIGEMM_STATUS_SUCCESS = 0,
+  CIGEMM_STATUS_NOT_INITIALIZED = 1,  /* null / destroyed handle                      */
+  CIGEMM_STATUS_ALLOC_FAILED = 3,
+  CIGEMM_STATUS_INVALID_VALUE = 7,    /* null pointer, negative size, ld too small ... */
+  CIGEMM_STATUS_ARCH_MISMATCH = 8,    /* device is not gfx950                          */
+  CIGEMM_STATUS_EXECUTION_FAILED = 13,/* HIP reported a launch / runtime error         */
+  CIGEMM_STATUS_INTERNAL_ERROR = 14,
+  CIGEMM_STATUS_NOT_SUPPORTED = 15    /* valid arguments, combination not implemented  */
+} cigemmStatus_t;
+
+/* Opaque library context (device, stream).  Takes the place of cublasHandle_t. */
+typedef struct cigemmContext* cigemmHandle_t;
+
+/* Layout of the second operand of the int8 GEMMs. */
+typedef enum cigemmBLayout {
+  CIGEMM_B_KN = 0, /* B is K x N row-major: C = A . B   (the reference's OP_N/OP_N case) */
+  CIGEMM_B_NK = 1  /* B is N x K row-major (weights, each output channel contiguous):
+                      C = A . B^T                                                      */
+} cigemmBLayout_t;
+
+typedef enum cigemmScaleMode {
+  CIGEMM_SCALE_TENSOR = 0, /* one float                                              */
+  CIGEMM_SCALE_VECTOR = 1  /* scaleA: one float per row of A (M); scaleB: one per
+                              column of C (N)                                         */
+} cigemmScaleMode_t;
+
+typedef enum cigemmOutType {
+  CIGEMM_OUT_F32 = 0,
+  CIGEMM_OUT_BF16 = 1
+} cigemmOutType_t;
+
+/* ---- lifecycle ------------------------------------------------------------------- */
+
+/* Replaces cublasCreate + cublasSetMathMode (quantization/main.cu:10-11).  Binds the
+ * handle to the current HIP device, which must be a gfx950; stream = the null stream. */
+CIGEMM_API cigemmStatus_t cigemmCreate(cigemmHandle_t* handle);
+
+/* Replaces cublasDestroy (quantization/main.cu:29). */
+CIGEMM_API cigemmStatus_t cigemmDestroy(cigemmHandle_t handle);
+
+/* Replaces cublasSetStream (implicit default stream in the reference).  `stream` is a
+ * hipStream_t passed as void*; NULL selects the null stream. */
+CIGEMM_API cigemmStatus_t cigemmSetStream(cigemmHandle_t handle, void* stream);
+CIGEMM_API cigemmStatus_t cigemmGetStream(cigemmHandle_t handle, void** stream);
+
+/* Replaces cublas_status_to_string (quantization/gemm_common.h:10-35). */
+CIGEMM_API const char* cigemmGetStatusString(cigemmStatus_t status);
+
+/* Text of the last error recorded on the handle ("" if none).  Valid until the next
+ * failing call on the same handle. */
+CIGEMM_API const char* cigemmGetLastErrorString(cigemmHandle_t handle);
+
+/* Library version, major*10000 + minor*100 + patch. */
+CIGEMM_API int cigemmGetVersion(void);
+
+/* Name of the kernel family the last successful GEMM call on this handle dispatched to
+ * (for tests and profiles), e.g. "bf16_mfma_256x256x64". */
+CIGEMM_API const char* cigemmGetLastKernelName(cigemmHandle_t handle);
+
+/* ---- GEMM: C[M x N] = A[M x K] . B[K x N], row-major ------------------------------- */
+
+/* Replaces cublasGemmEx(CUDA_R_32F x3, CUBLAS_COMPUTE_32F)
+ * (quantization/GEMM_fp32.cu:49-54, 62-67).  fp32 inputs, fp32 products and sums. */
+CIGEMM_API cigemmStatus_t cigemm_gemm_f32(cigemmHandle_t handle, int64_t M, int64_t N,
+                                          int64_t K, const float* A, int64_t lda,
+                                          const float* B, int64_t ldb, float* C, int64_t ldc);
+
+/* Replaces cublasGemmEx(CUDA_R_16F x3, CUBLAS_COMPUTE_32F)
+ * (quantization/GEMM_fp16.cu:51-56, 64-69).  IEEE binary16 in and out (uint16_t bit
+ * patterns), exact products, fp32 accumulation, one round-to-nearest-even narrowing. */
+CIGEMM_API cigemmStatus_t cigemm_gemm_f16(cigemmHandle_t handle, int64_t M, int64_t N,
+                                          int64_t K, const uint16_t* A, int64_t lda,
+                                          const uint16_t* B, int64_t ldb, uint16_t* C,
+                                          int64_t ldc);
+
+/* Replaces cublasGemmEx(CUDA_R_16BF x3, CUBLAS_COMPUTE_32F)
+ * (quantization/GEMM_bf16.cu:51-56, 64-69).  bfloat16 in and out, fp32 accumulation. */
+CIGEMM_API cigemmStatus_t cigemm_gemm_bf16(cigemmHandle_t handle, int64_t M, int64_t N,
+                                           int64_t K, const uint16_t* A, int64_t lda,
+                                           const uint16_t* B, int64_t ldb, uint16_t* C,
+                                           int64_t ldc);
+
+/* Replaces cublasGemmEx(CUDA_R_8I, CUDA_R_8I -> CUDA_R_32I, CUBLAS_COMPUTE_32I)
+ * (quantization/GEMM_int8.cu:51-56, 64-69): raw int32 accumulators out, exact. */
+CIGEMM_API cigemmStatus_t cigemm_gemm_i8_i32(cigemmHandle_t handle, int64_t M, int64_t N,
+                                             int64_t K, const int8_t* A, int64_t lda,
+                                             const int8_t* B, int64_t ldb,
+                                             cigemmBLayout_t b_layout, int32_t* C, int64_t ldc);
+
+/* int8 GEMM with the scale-and-dequantize epilogue fused into the kernel.  No reference
+ * counterpart (the reference stops at raw int32, quantization/GEMM_int8.cu:48-56); the
+ * epilogue is defined as
+ *     out[i][j] = ((float)acc[i][j] * scaleA[i or 0]) * scaleB[j or 0]
+ * evaluated left to right in fp32 without fusing, then (for CIGEMM_OUT_BF16) rounded to
+ * nearest even.  `out` is float* or uint16_t* according to `out_type`; `ldo` counts its
+ * elements.  `acc_out` may be NULL; otherwise the int32 accumulators are also stored
+ * there (leading dimension ldacc) by the same kernel. */
+CIGEMM_API cigemmStatus_t cigemm_gemm_i8_dequant(
+    cigemmHandle_t handle, int64_t M, int64_t N, int64_t K, const int8_t* A, int64_t lda,
+    const int8_t* B, int64_t ldb, cigemmBLayout_t b_layout, const float* scaleA,
+    cigemmScaleMode_t scaleA_mode, const float* scaleB, cigemmScaleMode_t scaleB_mode,
+    void* out, cigemmOutType_t out_type, int64_t ldo, int32_t* acc_out, int64_t ldacc);
+
+/* ---- device-side input generation -------------------------------------------------- */
+
+/* Replace fill_random_fp32 / _bf16 / _fp16 / _int8 (quantization/GEMM_fp32.cu:7-17,
+ * GEMM_bf16.cu:8-19, GEMM_fp16.cu:8-19, GEMM_int8.cu:8-19): element idx gets the value
+ * derived from ((idx ^ seed) * 2862933555777941757 + 3037000493) mod 2^64. */
+CIGEMM_API cigemmStatus_t cigemm_fill_random_f32(cigemmHandle_t handle, float* data,
+                                                 int64_t count, uint64_t seed, float lo,
+                                                 float hi);
+CIGEMM_API cigemmStatus_t cigemm_fill_random_bf16(cigemmHandle_t handle, uint16_t* data,
+                                                  int64_t count, uint64_t seed, float lo,
+                                                  float hi);
+CIGEMM_API cigemmStatus_t cigemm_fill_random_f16(cigemmHandle_t handle, uint16_t* data,
+                                                 int64_t count, uint64_t seed, float lo,
+                                                 float hi);
+CIGEMM_API cigemmStatus_t cigemm_fill_random_i8(cigemmHandle_t handle, int8_t* data,
+                                                int64_t count, uint64_t seed, int lo, int hi);
+
+/* ---- quantizer either side of the int8 GEMM ---------------------------------------- */
+
+/* Symmetric absmax int8 quantization of each row of x (rows x cols, fp32, row-major):
+ * scale[i] = absmax_i / 127 (1 when the row is all zero),
+ * q[i][j] = clamp(round-to-nearest-even(x[i][j] / scale[i]), -127, 127).
+ * No reference counterpart (the reference's quantization/ directory holds no quantizer);
+ * it prepares per-row activations and per-output-channel (N x K) weights. */
+CIGEMM_API cigemmStatus_t cigemm_quantize_rows_i8(cigemmHandle_t handle, int64_t rows,
+                                                  int64_t cols, const float* x, int64_t ldx,
+                                                  int8_t* q, int64_t ldq, float* scale);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CIGEMM_H_ */

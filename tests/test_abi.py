@@ -1,0 +1,82 @@
+"""The C-ABI library loads and exports exactly what include/cigemm.h declares.
+No compute call is made here (no GPU)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+import cudaintro_amd
+from cudaintro_amd import cigemm
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "cigemm.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"CIGEMM_API\s+[\w\s\*]+?\b(cigemm\w+)\s*\(", text)))
+
+
+def test_header_declares_expected_entry_points():
+    names = declared_symbols()
+    for must in ["cigemmCreate", "cigemmDestroy", "cigemmSetStream", "cigemm_gemm_f32",
+                 "cigemm_gemm_f16", "cigemm_gemm_bf16", "cigemm_gemm_i8_i32",
+                 "cigemm_gemm_i8_dequant", "cigemm_fill_random_i8", "cigemm_quantize_rows_i8"]:
+        assert must in names
+    assert len(names) >= 18
+
+
+def test_library_exports_every_declared_symbol():
+    lib = cudaintro_amd.load_library()
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in cigemm.h but not exported"
+
+
+def test_binding_covers_every_declared_symbol():
+    assert sorted(cigemm.SIGNATURES) == declared_symbols()
+
+
+def test_no_unexpected_exports():
+    """Only the C ABI is visible: no C++ symbols leak from the shared object."""
+    out = subprocess.run(["nm", "-D", "--defined-only", cudaintro_amd.library_path()],
+                         capture_output=True, text=True, check=True).stdout
+    exported = [l.split()[-1] for l in out.splitlines() if " T " in l]
+    assert sorted(exported) == declared_symbols()
+
+
+def test_header_compiles_as_c(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include "cigemm.h"\nint main(void){cigemmHandle_t h=0;(void)h;return CIGEMM_STATUS_SUCCESS;}\n')
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    "-c", str(src), "-o", str(tmp_path / "t.o")], check=True)
+
+
+def test_status_strings_and_null_handle():
+    lib = cudaintro_amd.load_library()
+    assert lib.cigemmGetStatusString(0) == b"CIGEMM_STATUS_SUCCESS"
+    assert lib.cigemmGetStatusString(7) == b"CIGEMM_STATUS_INVALID_VALUE"
+    assert lib.cigemmGetStatusString(99) == b"CIGEMM_STATUS_UNKNOWN"
+    assert lib.cigemmGetVersion() >= 100
+    # null handle: status code, never a crash
+    assert lib.cigemmDestroy(None) == cigemm.Status.NOT_INITIALIZED
+    assert lib.cigemmSetStream(None, None) == cigemm.Status.NOT_INITIALIZED
+    assert lib.cigemm_gemm_f32(None, 1, 1, 1, None, 1, None, 1, None, 1) == cigemm.Status.NOT_INITIALIZED
+    assert lib.cigemm_gemm_i8_i32(None, 1, 1, 1, None, 1, None, 1, 0, None, 1) == cigemm.Status.NOT_INITIALIZED
+    assert lib.cigemm_fill_random_f32(None, None, 0, 0, 0.0, 1.0) == cigemm.Status.NOT_INITIALIZED
+    assert lib.cigemmCreate(None) == cigemm.Status.INVALID_VALUE
+    assert lib.cigemmGetLastErrorString(None) == b""
+
+
+def test_create_fails_loudly_without_a_gpu():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    lib = cudaintro_amd.load_library()
+    h = ctypes.c_void_p()
+    st = lib.cigemmCreate(ctypes.byref(h))
+    assert st != 0 and not h.value
+    with pytest.raises(cudaintro_amd.CigemmError):
+        cudaintro_amd.Handle()

@@ -1,0 +1,93 @@
+"""fp32 GEMM through the C ABI against the reference CPU GEMM (oracle)."""
+import numpy as np
+import pytest
+
+from cudaintro_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 2, 3, 7, 17, 33, 65, 129]
+
+
+def run(handle, torch, A, B):
+    return handle.gemm_f32(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()).cpu().numpy()
+
+
+def scaled_tolerance_ok(gpu, cpu, tol=1e-5):
+    """|gpu - cpu| <= tol * max(|cpu|, rms(cpu)), every entry."""
+    rms = float(np.sqrt(np.mean(cpu.astype(np.float64) ** 2)))
+    lim = tol * np.maximum(np.abs(cpu.astype(np.float64)), rms)
+    err = np.abs(gpu.astype(np.float64) - cpu.astype(np.float64))
+    return bool((err <= lim).all()), float((err / lim).max())
+
+
+def test_config_fp32_512(handle, torch_gpu, oracle):
+    """fp32 512^3, U[-1,1], seed 0: within the 1e-5 scaled relative tolerance of the CPU loop."""
+    A, B = wl.fp32_uniform(512, 512, 512, seed=0)
+    C = run(handle, torch_gpu, A, B)
+    cpu = oracle.matrixMulCPU(A, B)
+    ok, worst = scaled_tolerance_ok(C, cpu)
+    assert ok, f"worst error {worst:.3f} x tolerance ({handle.last_kernel})"
+    # the GPU is no further from fp64 than the fp32 CPU loop's own bound
+    C64, S = oracle.gemm_f64(A, B, with_abs=True)
+    assert (np.abs(C - C64) <= 512 * 2.0 ** -24 * S).all()
+
+
+@pytest.mark.parametrize("M", SIZES)
+@pytest.mark.parametrize("N,K", [(1, 1), (3, 129), (17, 7), (33, 65), (129, 33), (65, 2)])
+def test_ragged_shapes(handle, torch_gpu, oracle, rng, M, N, K):
+    A = rng.uniform(-1, 1, size=(M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, size=(K, N)).astype(np.float32)
+    C = run(handle, torch_gpu, A, B)
+    cpu = oracle.gemm_f32(A, B)
+    ok, worst = scaled_tolerance_ok(C, cpu)
+    assert ok, f"{M}x{N}x{K}: {worst}"
+
+
+def test_exact_inputs_are_bit_exact(handle, torch_gpu, oracle, rng):
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    for (M, N, K) in [(64, 64, 64), (256, 256, 256), (130, 70, 1000), (512, 512, 512)]:
+        A = rng.choice(vals, size=(M, K))
+        B = rng.choice(vals, size=(K, N))
+        np.testing.assert_array_equal(run(handle, torch_gpu, A, B), oracle.gemm_f32(A, B))
+
+
+def test_identity_onehot_leading_dims(handle, torch_gpu, oracle, rng):
+    torch = torch_gpu
+    n = 96
+    A = rng.normal(size=(n, n)).astype(np.float32)
+    I = np.eye(n, dtype=np.float32)
+    np.testing.assert_array_equal(run(handle, torch, A, I), A)
+    np.testing.assert_array_equal(run(handle, torch, I, A), A)
+    # ld > cols: operate on sub-blocks of larger device buffers, output into a padded buffer
+    big_a = torch.from_numpy(rng.normal(size=(50, 100)).astype(np.float32)).cuda()
+    big_b = torch.from_numpy(rng.normal(size=(70, 90)).astype(np.float32)).cuda()
+    out = torch.full((50, 64), -7.0, dtype=torch.float32, device="cuda")
+    a, b, c = big_a[:, 10:80], big_b[:, 5:45], out[:, 3:43]
+    handle.gemm_f32(a, b, out=c)
+    cpu = oracle.gemm_f32(a.cpu().numpy(), b.cpu().numpy())
+    ok, worst = scaled_tolerance_ok(c.cpu().numpy(), cpu)
+    assert ok, worst
+    o = out.cpu().numpy()
+    assert (o[:, :3] == -7.0).all() and (o[:, 43:] == -7.0).all()   # nothing outside C touched
+
+
+def test_generic_kernel_equals_cpu_loop_bit_for_bit(handle, torch_gpu, oracle, rng):
+    """The any-shape kernel adds one separately rounded product at a time in ascending k,
+    the same order as the reference CPU loop."""
+    A = rng.uniform(-1, 1, size=(77, 300)).astype(np.float32)
+    B = rng.uniform(-1, 1, size=(300, 91)).astype(np.float32)
+    C = run(handle, torch_gpu, A, B)
+    assert "generic" in handle.last_kernel
+    np.testing.assert_array_equal(C, oracle.gemm_f32(A, B))
+
+
+def test_k_zero_and_empty(handle, torch_gpu):
+    torch = torch_gpu
+    A = torch.empty((4, 0), dtype=torch.float32, device="cuda")
+    B = torch.empty((0, 5), dtype=torch.float32, device="cuda")
+    out = torch.full((4, 5), 3.0, dtype=torch.float32, device="cuda")
+    handle.gemm_f32(A, B, out=out)
+    assert (out.cpu().numpy() == 0).all()          # empty sum
+    handle.gemm_f32(torch.empty((0, 3), dtype=torch.float32, device="cuda"),
+                    torch.empty((3, 5), dtype=torch.float32, device="cuda"))

@@ -1,0 +1,25 @@
+"""Builds and runs the C++ host-logic test (timing protocol with a fake clock, driver
+stdout formats, GemmResult layout) with the host compiler; no GPU involved."""
+import os
+import subprocess
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_host_protocol(tmp_path):
+    exe = tmp_path / "test_host_protocol"
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-D__HIP_PLATFORM_AMD__",
+                    "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "cudaintro_amd", "csrc"),
+                    "-I", "/opt/rocm/include", os.path.join(ROOT, "tests", "cpp", "test_host_protocol.cpp"),
+                    "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "host protocol OK" in out.stdout
+
+
+def test_gemm_common_header_names():
+    """The drop-in header keeps the record and the four entry-point names."""
+    text = open(os.path.join(ROOT, "include", "gemm_common.h")).read()
+    for name in ("struct GemmResult", "run_gemm_bf16", "run_gemm_fp16", "run_gemm_fp32", "run_gemm_int8",
+                 "const char* name;", "uint64_t iters;", "double secs;", "double tflops;"):
+        assert name in text
