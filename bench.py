@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X quantization-GEMM library.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+
+Headline (the one JSON line printed last): bf16 GEMM 8192^3, TFLOP/s = 2*M*N*K / time, inputs
+resident in HBM before the timed region; one "step" is one GEMM call.  The same line carries
+`per_config` (fp16 and int8 at 8192^3, int8 4096^3 with per-tensor dequant, the quantized
+linear prefill shape, the skinny decode shapes in GB/s), the `roofline` of the headline
+kernel (HIP-event timed on the launch stream) and the `cpu_baseline` (the CPU port of the
+reference triple loop timed on a bounded slice of rows of the same problem).
+
+One GPU only: --gpus above 1 exits with a message.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published dense peaks: 256 CUs x 4 SIMDs x 2.4 GHz x 1024 flop/clk (16-bit), x2 for int8.
+PEAK_16BIT_TFLOPS = 2516.6
+PEAK_INT8_TOPS = 5033.2
+PEAK_FP32_MATRIX_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_calls(torch, fn, steps, warmup):
+    """W untimed calls, then exactly `steps` calls between a synchronize on both sides.
+    Returns (wall seconds, HIP-event seconds) for the timed region."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, e0.elapsed_time(e1) * 1e-3
+
+
+def dev16(torch, bits, kind):
+    if kind == "bf16":
+        return torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(bits.view(np.float16)).cuda()
+
+
+def cpu_baseline_16bit(Ab, Bb, kind, target_seconds=12.0):
+    """The CPU port of the reference triple loop (i-j-k, float accumulator) on the first R
+    rows of the same problem; cost is exactly linear in rows."""
+    import oracle
+    from cudaintro_amd import workloads as wl
+    A = wl.widen_16bit(Ab, kind)
+    B = wl.widen_16bit(Bb, kind)
+    M, K = A.shape
+    N = B.shape[1]
+    threads = oracle.num_threads()
+    rows = max(threads, 16)
+    probe = np.empty((rows, N), np.float32)
+    t0 = time.perf_counter()
+    oracle.lib.oracle_gemm_f32_ijk(M, N, K, A.ctypes.data, K, B.ctypes.data, N, probe.ctypes.data,
+                                   N, 0, rows)
+    dt = time.perf_counter() - t0
+    scale = max(1, int(target_seconds / max(dt, 1e-3)))
+    rows2 = min(M, rows * scale)
+    rows2 -= rows2 % threads
+    rows2 = max(rows2, threads)
+    out = np.empty((rows2, N), np.float32)
+    t0 = time.perf_counter()
+    oracle.lib.oracle_gemm_f32_ijk(M, N, K, A.ctypes.data, K, B.ctypes.data, N, out.ctypes.data, N,
+                                   0, rows2)
+    dt = time.perf_counter() - t0
+    tflops = 2.0 * rows2 * N * K / dt / 1e12
+    return {"value": tflops, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"first {rows2} of {M} rows of the same {M}x{N}x{K} problem, "
+                      f"fp32 i-j-k triple loop, {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-extra", action="store_true", help="headline workload only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--size", type=int, default=8192, help="headline M=N=K (default 8192)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import cudaintro_amd as ci
+    from cudaintro_amd import workloads as wl
+
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X; there is no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    handle = ci.Handle()
+    n = args.size
+    per_config = {}
+
+    # ---- headline: bf16 n^3 -------------------------------------------------------------
+    log(f"[bench] generating bf16 {n}^3 inputs")
+    Ab, Bb = wl.normal_16bit(n, n, n, seed=2, kind="bf16")
+    A, B = dev16(torch, Ab, "bf16"), dev16(torch, Bb, "bf16")
+    C = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
+    wall, ev = time_calls(torch, lambda: handle.gemm_bf16(A, B, out=C), args.steps, args.warmup)
+    kernel = handle.last_kernel
+    ops = wl.gemm_ops(n, n, n)
+    value = ops * args.steps / wall / 1e12
+    achieved = ops * args.steps / ev / 1e12
+    log(f"[bench] bf16 {n}^3: {value:.1f} TFLOP/s wall, {achieved:.1f} TFLOP/s by HIP events, "
+        f"kernel {kernel}")
+    roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_16BIT_TFLOPS, "unit": "TFLOP/s",
+                "frac": achieved / PEAK_16BIT_TFLOPS, "traffic": None, "kernel": kernel,
+                "avg_kernel_ms": ev / args.steps * 1e3}
+    traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(traffic_file):
+        roofline["traffic"] = json.load(open(traffic_file)).get(f"bf16_{n}")
+
+    cpu = None
+    if not args.no_cpu:
+        log("[bench] CPU baseline (port of the reference triple loop) ...")
+        cpu = cpu_baseline_16bit(Ab, Bb, "bf16")
+        log(f"[bench] CPU: {cpu['value'] * 1e3:.2f} GFLOP/s on {cpu['cores']} threads")
+    del A, B, C
+
+    if not args.no_extra:
+        def run16(kind):
+            a_b, b_b = wl.normal_16bit(n, n, n, seed=2, kind=kind)
+            a, b = dev16(torch, a_b, kind), dev16(torch, b_b, kind)
+            c = torch.empty((n, n), dtype=a.dtype, device="cuda")
+            fn = handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16
+            w, e = time_calls(torch, lambda: fn(a, b, out=c), args.steps, args.warmup)
+            t = ops * args.steps / e / 1e12
+            return {"tflops": t, "frac_of_peak": t / PEAK_16BIT_TFLOPS, "peak": PEAK_16BIT_TFLOPS,
+                    "ms": e / args.steps * 1e3, "kernel": handle.last_kernel}
+
+        log(f"[bench] fp16 {n}^3")
+        per_config[f"fp16_{n}"] = run16("f16")
+        per_config[f"bf16_{n}"] = {"tflops": achieved, "frac_of_peak": achieved / PEAK_16BIT_TFLOPS,
+                                   "peak": PEAK_16BIT_TFLOPS, "ms": ev / args.steps * 1e3,
+                                   "kernel": kernel}
+
+        def run_i8(name, M, N, K, make, dequant):
+            log(f"[bench] {name}")
+            Aq, Bq, sa, sb, lay, out_t = make()
+            a, b = torch.from_numpy(Aq).cuda(), torch.from_numpy(Bq).cuda()
+            if dequant:
+                sa_d, sb_d = torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda()
+                out = torch.empty((M, N), device="cuda",
+                                  dtype=torch.bfloat16 if out_t == ci.OUT_BF16 else torch.float32)
+                fn = lambda: handle.gemm_i8_dequant(a, b, sa_d, sb_d, lay, out_t, out=out)  # noqa: E731
+            else:
+                out = torch.empty((M, N), dtype=torch.int32, device="cuda")
+                fn = lambda: handle.gemm_i8_i32(a, b, lay, out=out)  # noqa: E731
+            w, e = time_calls(torch, fn, args.steps, args.warmup)
+            t = wl.gemm_ops(M, N, K) * args.steps / e / 1e12
+            per_config[name] = {"tops": t, "frac_of_peak": t / PEAK_INT8_TOPS, "peak": PEAK_INT8_TOPS,
+                                "ms": e / args.steps * 1e3, "kernel": handle.last_kernel}
+
+        def mk_square(sz, seed):
+            def f():
+                Aq, Bq, sa, sb = wl.int8_uniform(sz, sz, sz, seed=seed)
+                return Aq, Bq, sa, sb, ci.B_KN, ci.OUT_F32
+            return f
+
+        def mk_linear():
+            Xq, sx, Wq, sw = wl.quantized_linear(2048, 4096, 11008, seed=3)
+            return Xq, Wq, sx, sw, ci.B_NK, ci.OUT_BF16
+
+        run_i8(f"int8_{n}_raw_i32", n, n, n, mk_square(n, 1), False)
+        run_i8("int8_4096_dequant_f32", 4096, 4096, 4096, mk_square(4096, 1), True)
+        run_i8("int8_linear_2048x11008x4096_dequant_bf16", 2048, 11008, 4096, mk_linear, True)
+
+        # fp32 anchor and the reference's own 4096^3
+        for sz in (512, 4096):
+            Af, Bf = wl.fp32_uniform(sz, sz, sz, seed=0)
+            a, b = torch.from_numpy(Af).cuda(), torch.from_numpy(Bf).cuda()
+            c = torch.empty((sz, sz), dtype=torch.float32, device="cuda")
+            steps = args.steps if sz == 512 else max(2, args.steps // 4)
+            w, e = time_calls(torch, lambda: handle.gemm_f32(a, b, out=c), steps, 2)
+            t = wl.gemm_ops(sz, sz, sz) * steps / e / 1e12
+            per_config[f"fp32_{sz}"] = {"tflops": t, "frac_of_peak": t / PEAK_FP32_MATRIX_TFLOPS,
+                                        "peak": PEAK_FP32_MATRIX_TFLOPS, "ms": e / steps * 1e3,
+                                        "kernel": handle.last_kernel}
+
+        # skinny decode shapes: HBM-bound.  Rotate over several distinct weight buffers so the
+        # working set (> 256 MB) cannot sit in the Infinity Cache between calls.
+        for M in (1, 8, 32):
+            xb, wb = wl.skinny_bf16(M, 8192, 8192, seed=4)
+            x = dev16(torch, xb, "bf16")
+            ws = [dev16(torch, wb, "bf16") for _ in range(4)]
+            y = torch.empty((M, 8192), dtype=torch.bfloat16, device="cuda")
+            it = [0]
+
+            def fn():
+                handle.gemm_bf16(x, ws[it[0] & 3], out=y)
+                it[0] += 1
+            steps = max(args.steps, 40)
+            w, e = time_calls(torch, fn, steps, 4)
+            nbytes = wl.skinny_bytes(M, 8192, 8192, 2, 2, 2)
+            gbs = nbytes * steps / e / 1e9
+            per_config[f"skinny_bf16_M{M}"] = {"gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS,
+                                               "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
+                                               "bytes": nbytes, "kernel": handle.last_kernel}
+            del ws
+            xq, sx, wq, sw = wl.skinny_int8(M, 8192, 8192, seed=4)
+            xd, sxd, swd = torch.from_numpy(xq).cuda(), torch.from_numpy(sx).cuda(), torch.from_numpy(sw).cuda()
+            wqs = [torch.from_numpy(wq).cuda() for _ in range(6)]
+            yo = torch.empty((M, 8192), dtype=torch.bfloat16, device="cuda")
+
+            def fn8():
+                handle.gemm_i8_dequant(xd, wqs[it[0] % 6], sxd, swd, ci.B_NK, ci.OUT_BF16, out=yo)
+                it[0] += 1
+            w, e = time_calls(torch, fn8, steps, 6)
+            nbytes = wl.skinny_bytes(M, 8192, 8192, 1, 1, 2, scale_bytes=4 * 8192)
+            gbs = nbytes * steps / e / 1e9
+            per_config[f"skinny_int8_M{M}"] = {"gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS,
+                                               "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
+                                               "bytes": nbytes, "kernel": handle.last_kernel}
+            del wqs
+        for k, v in per_config.items():
+            log(f"[bench]   {k}: {json.dumps(v)}")
+
+    line = {
+        "metric": "GEMM TFLOPS/TOPS at 8192^3 per dtype (int8/bf16/fp16) + % of MFMA peak",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"bf16 GEMM M=N=K={n}, N(0,1) inputs rounded to bf16, fp32 accumulate, "
+                               "bf16 out, row-major", "M": n, "N": n, "K": n},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "per_config": per_config,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
