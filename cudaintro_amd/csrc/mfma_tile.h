@@ -2,7 +2,14 @@
 //
 // Workgroup = 256 lanes = 4 waves (2 x 2); macro tile 256 (m) x 256 (n) x 128 BYTES of k
 // (64 halves or 128 int8).  Each wave owns a 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32
-// = 256 accumulators per lane.  Both operand tiles are 32 KiB; two stages are kept in LDS.
+// = 256 accumulators per lane (the AGPR file); one wave per SIMD.  Both operand tiles are
+// 32 KiB; two stages are kept in LDS (128 of the 160 KiB).
+//
+// Global -> LDS goes straight through the LDS-DMA path (global_load_lds_dwordx4): no
+// staging registers, no ds_write.  One such instruction deposits the wave's 64 x 16 bytes
+// contiguously in LDS, lane by lane, while each lane chooses its own global address; the
+// bank-conflict swizzle is therefore applied on the global side (the chunk a lane fetches),
+// and LDS slot s of a row holds chunk s ^ swizzle(row).
 //
 // A tile  [256 m][128 B of k], as in memory.  16-byte chunk c of row r lives at
 //         r*128 + ((c ^ fA(r)) << 4): the 16-byte fragment reads of 32 consecutive rows
@@ -15,6 +22,12 @@
 //         address of 8 bytes of row k0 + i/4 (i/2 for bytes) and receives the 4 (8)
 //         k-values of column n0 + i.  Chunks are XOR-swizzled by k so that the rows one
 //         instruction touches fall in different banks.
+//
+// Pipeline (per 128-byte k stage = 4 MFMA k-steps of 16 MFMAs each): fragments are double
+// buffered in registers, the reads of k-step s+1 are issued under the MFMAs of k-step s.
+// After k-step 2 the wave waits for its DMA of the next stage, crosses the single barrier
+// of the iteration, issues the DMA of the stage after next into the buffer just drained,
+// and reads the first fragments of the next stage under the MFMAs of k-step 3.
 //
 // The MFMA is issued with the B fragment as its first operand and the A fragment as its
 // second, so it yields the transposed 32 x 32 block: lane l holds, for the single output
@@ -37,11 +50,13 @@ constexpr int LDS_BYTES = 2 * STAGE_BYTES;  // 128 KiB of the 160 KiB
 
 typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) void global_void;
 
 // ---- A-like tile: [256 rows][8 chunks] ----------------------------------------------------
+__device__ __forceinline__ int rowmajor_swz(int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); }
 __device__ __forceinline__ int rowmajor_off(int r, int c) {
-  const int f = ((r >> 1) & 7) ^ ((r & 1) << 2);
-  return r * KB + ((c ^ f) << 4);
+  return r * KB + ((c ^ rowmajor_swz(r)) << 4);
 }
 
 enum BMode { B_NK = 0, B_KN16 = 1, B_KN8 = 2 };
@@ -49,65 +64,72 @@ enum BMode { B_NK = 0, B_KN16 = 1, B_KN8 = 2 };
 template <int MODE>
 struct BTile;
 
+// DMA geometry of a tile: wave w issues instruction i (0..7); the instruction fills 1 KiB of
+// LDS starting at dma_lds(w, i); lane l fetches the 16 bytes at global byte offset
+// dma_src(w, i, l, ld) from the tile's origin (row stride ld bytes).
+
+// [256 rows][128 B]: one instruction = 8 rows.
+struct RowMajorDma {
+  static __device__ __forceinline__ int dma_lds(int w, int i) { return (64 * w + 8 * i) * KB; }
+  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
+    const int r = 64 * w + 8 * i + (l >> 3);
+    return (int64_t)r * ld + (((l & 7) ^ rowmajor_swz(r)) << 4);
+  }
+};
+
 // Weights N x K: identical to the A tile.
 template <>
-struct BTile<B_NK> {
-  // lane t loads chunk t%8 of row t/8 + 32 i
-  static __device__ __forceinline__ int ld_row(int t, int i) { return (t >> 3) + 32 * i; }
-  static __device__ __forceinline__ int ld_chunk(int t) { return t & 7; }
-  static __device__ __forceinline__ int off(int r, int c) { return rowmajor_off(r, c); }
-  // global element offset of (tile row r = n, chunk c) at k byte offset kbyte0
-  static __device__ __forceinline__ int64_t gofs(int r, int c, int64_t ld, int64_t n0,
-                                                 int64_t kbyte0) {
-    return (n0 + r) * ld + kbyte0 + c * 16;  // bytes == elements (int8)
-  }
-  // fragment for column tile j of wave column wn, k-step kk
-  static __device__ __forceinline__ u32x4 frag(const char* sb, int wn, int j, int kk, int l) {
+struct BTile<B_NK> : RowMajorDma {
+  // half h (0/1) of the fragment of column tile j, k-step kk: 8 bytes of k
+  static __device__ __forceinline__ u32x2 frag_half(const char* sb, int wn, int j, int kk, int h,
+                                                    int l) {
     const int r = wn * 128 + 32 * j + (l & 31);
-    return *reinterpret_cast<const u32x4*>(sb + rowmajor_off(r, 2 * kk + (l >> 5)));
+    return *reinterpret_cast<const u32x2*>(sb + rowmajor_off(r, 2 * kk + (l >> 5)) + 8 * h);
   }
 };
 
-// K x N halves: [64 k][32 chunks of 8 halves].
+// K x N halves: [64 k][32 chunks of 8 halves]; one DMA instruction = 2 k-rows.
 template <>
 struct BTile<B_KN16> {
-  static __device__ __forceinline__ int ld_row(int t, int i) { return (t >> 5) + 8 * i; }
-  static __device__ __forceinline__ int ld_chunk(int t) { return t & 31; }
-  static __device__ __forceinline__ int off(int k, int c) {
+  static __device__ __forceinline__ int swz(int k) {
     const int k3 = k & 3;
-    const int g = (k3 << 2) | ((((k3 >> 1) ^ k3) & 1) << 1);
-    return k * 512 + ((c ^ g) << 4);
+    return (k3 << 2) | ((((k3 >> 1) ^ k3) & 1) << 1);
   }
-  static __device__ __forceinline__ u32x4 frag(const char* sb, int wn, int j, int kk, int l) {
-    const int k_lo = 16 * kk + 8 * (l >> 5) + ((l & 15) >> 2);
+  static __device__ __forceinline__ int off(int k, int c) { return k * 512 + ((c ^ swz(k)) << 4); }
+  static __device__ __forceinline__ int dma_lds(int w, int i) { return (16 * w + 2 * i) * 512; }
+  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
+    const int k = 16 * w + 2 * i + (l >> 5);
+    return (int64_t)k * ld + (((l & 31) ^ swz(k)) << 4);
+  }
+  static __device__ __forceinline__ u32x2 frag_half(const char* sb, int wn, int j, int kk, int h,
+                                                    int l) {
+    const int k = 16 * kk + 8 * (l >> 5) + ((l & 15) >> 2) + 4 * h;
     const int n = wn * 128 + 32 * j + 16 * ((l >> 4) & 1) + 4 * (l & 3);
     const int sub = ((n >> 2) & 1) * 8;
-    i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(sb + off(k_lo, n >> 3) + sub));
-    i16x4 hi =
-        __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(sb + off(k_lo + 4, n >> 3) + sub));
-    i16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(u32x4, both);
+    i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(sb + off(k, n >> 3) + sub));
+    return __builtin_bit_cast(u32x2, v);
   }
 };
 
-// K x N bytes: [128 k][16 chunks of 16 bytes].
+// K x N bytes: [128 k][16 chunks of 16 bytes]; one DMA instruction = 4 k-rows.
 template <>
 struct BTile<B_KN8> {
-  static __device__ __forceinline__ int ld_row(int t, int i) { return (t >> 4) + 16 * i; }
-  static __device__ __forceinline__ int ld_chunk(int t) { return t & 15; }
-  static __device__ __forceinline__ int off(int k, int c) {
-    const int g = ((k & 7) << 1) | (((k >> 2) ^ (k >> 4)) & 1);
-    return k * 256 + ((c ^ g) << 4);
+  static __device__ __forceinline__ int swz(int k) {
+    return ((k & 7) << 1) | (((k >> 2) ^ (k >> 4)) & 1);
   }
-  static __device__ __forceinline__ u32x4 frag(const char* sb, int wn, int j, int kk, int l) {
-    const int k_lo = 32 * kk + 16 * (l >> 5) + ((l & 15) >> 1);
+  static __device__ __forceinline__ int off(int k, int c) { return k * 256 + ((c ^ swz(k)) << 4); }
+  static __device__ __forceinline__ int dma_lds(int w, int i) { return (32 * w + 4 * i) * 256; }
+  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
+    const int k = 32 * w + 4 * i + (l >> 4);
+    return (int64_t)k * ld + (((l & 15) ^ swz(k)) << 4);
+  }
+  static __device__ __forceinline__ u32x2 frag_half(const char* sb, int wn, int j, int kk, int h,
+                                                    int l) {
+    const int k = 32 * kk + 16 * (l >> 5) + ((l & 15) >> 1) + 8 * h;
     const int n = wn * 128 + 32 * j + 16 * ((l >> 4) & 1) + 8 * (l & 1);
     const int sub = ((n >> 3) & 1) * 8;
-    i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(sb + off(k_lo, n >> 4) + sub));
-    i32x2 hi =
-        __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(sb + off(k_lo + 8, n >> 4) + sub));
-    i32x4 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
-    return __builtin_bit_cast(u32x4, both);
+    i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(sb + off(k, n >> 4) + sub));
+    return __builtin_bit_cast(u32x2, v);
   }
 };
 
@@ -177,56 +199,69 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int t = threadIdx.x;
   const int l = t & 63;
-  const int w = t >> 6;
+  const int w = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wm = w >> 1, wn = w & 1;
 
   int tm, tn;
   tile_of_workgroup(tiles_m, tiles_n, tm, tn);
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
 
-  // ---- global -> register staging: 8 + 8 16-byte loads per lane per stage -------------------
-  const int a_chunk = t & 7;
-  const char* a_src = A + (m0 + (t >> 3)) * lda + a_chunk * 16;
-  const int64_t a_step = 32 * lda;  // between this lane's 8 rows
-  const char* b_src;
-  int64_t b_step, b_kstep;  // between this lane's 8 rows; between stages
+  // ---- DMA sources: uniform tile origin + per-lane 32-bit byte offsets ----------------------
+  const char* a_tile = A + m0 * lda;  // + kt * KB
+  const char* b_tile;                 // + kt * b_kstep
+  int64_t b_kstep;
   if (BMODE == B_NK) {
-    b_src = B + (n0 + BT::ld_row(t, 0)) * ldb + BT::ld_chunk(t) * 16;
-    b_step = 32 * ldb;
+    b_tile = B + n0 * ldb;
     b_kstep = KB;
   } else {
-    b_src = B + (int64_t)BT::ld_row(t, 0) * ldb + n0 * Math::ELEM_BYTES + BT::ld_chunk(t) * 16;
-    b_step = (int64_t)(BT::ld_row(t, 1) - BT::ld_row(t, 0)) * ldb;
+    b_tile = B + n0 * Math::ELEM_BYTES;
     b_kstep = (int64_t)(KB / Math::ELEM_BYTES) * ldb;
   }
-  int a_dst[8], b_dst[8];
+  uint32_t a_voff[8], b_voff[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    a_dst[i] = rowmajor_off((t >> 3) + 32 * i, a_chunk);
-    b_dst[i] = OPERAND_BYTES + BT::off(BT::ld_row(t, i), BT::ld_chunk(t));
+    a_voff[i] = (uint32_t)RowMajorDma::dma_src(w, i, l, lda);
+    b_voff[i] = (uint32_t)BT::dma_src(w, i, l, ldb);
   }
-  u32x4 a_stage[8], b_stage[8];
 
-  auto load_global = [&](int kt) {
-    const char* ap = a_src + (int64_t)kt * KB;
-    const char* bp = b_src + (int64_t)kt * b_kstep;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      a_stage[i] = *reinterpret_cast<const u32x4*>(ap + i * a_step);
-      b_stage[i] = *reinterpret_cast<const u32x4*>(bp + i * b_step);
-    }
+  // The DMA instructions are written as asm so that the compiler's wait-count insertion does
+  // not know them: it would otherwise make every later LDS read it cannot tell apart (the
+  // transposing reads) wait for all outstanding DMA.  Completion is waited for by hand
+  // (vmcnt) before the barrier that publishes a stage.  M0 carries the wave-uniform LDS
+  // destination; lane l's 16 bytes land at M0 + 16 l.
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  auto dma16 = [&](const char* src, uint32_t lds_dst) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_dst), "v"(src)
+                 : "m0");
   };
-  auto store_lds = [&](int buf) {
-    char* base = lds + buf * STAGE_BYTES;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      *reinterpret_cast<u32x4*>(base + a_dst[i]) = a_stage[i];
-      *reinterpret_cast<u32x4*>(base + b_dst[i]) = b_stage[i];
-    }
+  // DMA instruction d (0..15) of a stage: even d = A piece d/2, odd d = B piece d/2.
+  auto dma_piece = [&](int kt, int buf, int d) {
+    const uint32_t sa = lds_base + buf * STAGE_BYTES;
+    const int i = d >> 1;
+    if (d & 1)
+      dma16(b_tile + (int64_t)kt * b_kstep + b_voff[i], sa + OPERAND_BYTES + BT::dma_lds(w, i));
+    else
+      dma16(a_tile + (int64_t)kt * KB + a_voff[i], sa + RowMajorDma::dma_lds(w, i));
   };
 
   const int a_frag_row = wm * 128 + (l & 31);
   const int g = l >> 5;
+
+  // One k-step's operands: 4 A fragments (16 B each) and 4 B fragments as 8 halves.
+  struct Frags {
+    u32x4 a[4];
+    u32x2 b[8];
+  };
+  // LDS read r (0..11) of k-step kk of the stage in `buf`: 0..3 = A fragment r, 4..11 = B half.
+  auto read_piece = [&](Frags& f, int buf, int kk, int r) {
+    const char* sa = lds + buf * STAGE_BYTES;
+    if (r < 4)
+      f.a[r] = *reinterpret_cast<const u32x4*>(sa + rowmajor_off(a_frag_row + 32 * r, 2 * kk + g));
+    else
+      f.b[r - 4] = BT::frag_half(sa + OPERAND_BYTES, wn, (r - 4) >> 1, kk, (r - 4) & 1, l);
+  };
 
   acc_t acc[4][4];
 #pragma unroll
@@ -236,31 +271,59 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
+  // MFMA m (0..15) of a k-step, column tile j = m/4 outer: the first four need all A
+  // fragments (reads 0..3) but only the first B fragment (reads 4, 5).
+  auto mfma_piece = [&](const Frags& f, int m) {
+    const int j = m >> 2, i = m & 3;
+    const u32x4 bfrag = __builtin_shufflevector(f.b[2 * j], f.b[2 * j + 1], 0, 1, 2, 3);
+    acc[i][j] = Math::mfma(bfrag, f.a[i], acc[i][j]);
+  };
+
+  Frags f0, f1;
+
+  // prologue: stages 0 and 1 in flight, first fragments in registers
+#pragma unroll
+  for (int d = 0; d < 16; ++d) dma_piece(0, 0, d);
+  if (KT > 1) {
+#pragma unroll
+    for (int d = 0; d < 16; ++d) dma_piece(1, 1, d);
+    __builtin_amdgcn_s_waitcnt(0x4f70);  // vmcnt(16): stage 0 landed, stage 1 may be in flight
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  }
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int r = 0; r < 12; ++r) read_piece(f0, 0, 0, r);
+
+  // One k-step: 16 slots, each one MFMA on `cur` plus at most one LDS read into `nxt` (the
+  // operands of the following k-step) and at most one DMA instruction; the fences keep the
+  // emitted order equal to this one.
+#define CIG_KSTEP(cur, nxt, rbuf, rkk, WITH_DMA, dkt, dbuf)          \
+  _Pragma("unroll") for (int sl = 0; sl < 16; ++sl) {                \
+    mfma_piece(cur, sl);                                             \
+    if (sl < 12) read_piece(nxt, rbuf, rkk, sl);                     \
+    if (WITH_DMA) dma_piece(dkt, dbuf, sl);                          \
+    __builtin_amdgcn_sched_barrier(0);                               \
+  }
 
   for (int kt = 0; kt < KT; ++kt) {
     const int buf = kt & 1;
-    if (kt + 1 < KT) load_global(kt + 1);
-    const char* sa = lds + buf * STAGE_BYTES;
-    const char* sb = sa + OPERAND_BYTES;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      u32x4 af[4], bf[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        af[i] = *reinterpret_cast<const u32x4*>(sa + rowmajor_off(a_frag_row + 32 * i, 2 * kk + g));
-#pragma unroll
-      for (int j = 0; j < 4; ++j) bf[j] = BT::frag(sb, wn, j, kk, l);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = Math::mfma(bf[j], af[i], acc[i][j]);
-    }
-    if (kt + 1 < KT) store_lds(buf ^ 1);
-    __syncthreads();
+    CIG_KSTEP(f0, f1, buf, 1, false, 0, 0);  // MFMA (kt,0), read (kt,1)
+    CIG_KSTEP(f1, f0, buf, 2, false, 0, 0);  // MFMA (kt,1), read (kt,2)
+    CIG_KSTEP(f0, f1, buf, 3, false, 0, 0);  // MFMA (kt,2), read (kt,3)
+    // stage kt fully read by this wave; stage kt+1 must have landed for everybody
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // Branch-free so the iteration stays straight-line code: past the end the last stage is
+    // fetched again into the buffer nobody reads any more, and the fragment reads of the
+    // (non-existent) next stage are harmless LDS reads.
+    const int knext = kt + 2 < KT ? kt + 2 : KT - 1;
+    CIG_KSTEP(f1, f0, buf ^ 1, 0, true, knext, buf);  // MFMA (kt,3), read (kt+1,0), DMA kt+2
   }
+#undef CIG_KSTEP
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): no DMA outlives the main loop
 
   // acc[i][j][4q+e] = C[m0 + wm*128 + 32i + l%32][n0 + wn*128 + 32j + 8q + 4g + e]
 #pragma unroll
@@ -292,6 +355,7 @@ void launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
 }
 
 // Shape / alignment gate shared by the families (sizes in elements, elem = bytes each).
+// Per-lane DMA offsets are 32-bit: 256 rows of either operand must span less than 4 GiB.
 inline bool tile_shape_ok(int64_t M, int64_t N, int64_t K, int elem, const void* A, int64_t lda,
                           const void* B, int64_t ldb) {
   if (M <= 0 || N <= 0 || K <= 0) return false;
@@ -299,6 +363,7 @@ inline bool tile_shape_ok(int64_t M, int64_t N, int64_t K, int elem, const void*
   if ((lda * elem) % 16 || (ldb * elem) % 16) return false;
   if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return false;
   if ((M / BM) * (N / BN) > 2147483647LL) return false;
+  if (lda * elem * 256 >= (1LL << 32) || ldb * elem * 256 >= (1LL << 32)) return false;
   return true;
 }
 
