@@ -31,11 +31,11 @@ bool launch_16b_mfma(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_
   if (bf16) {
     tile::launch_tile<tile::MathBF16, tile::B_KN16>(ctx, M, N, K * 2, A, lda * 2, B, ldb * 2,
                                                     EpiStore16x4<BF16>{C, ldc});
-    ctx->last_kernel = "bf16_mfma_256x256x64";
+    ctx->last_kernel = "bf16_mfma_256x256x32_ring4";
   } else {
     tile::launch_tile<tile::MathF16, tile::B_KN16>(ctx, M, N, K * 2, A, lda * 2, B, ldb * 2,
                                                    EpiStore16x4<F16>{C, ldc});
-    ctx->last_kernel = "f16_mfma_256x256x64";
+    ctx->last_kernel = "f16_mfma_256x256x32_ring4";
   }
   return true;
 }

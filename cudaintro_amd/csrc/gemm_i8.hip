@@ -97,8 +97,8 @@ bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const i
     launch_layout<tile::B_NK>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
   else
     launch_layout<tile::B_KN8>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
-  ctx->last_kernel = dq ? (b_nk ? "i8_mfma_256x256x128_nk_dequant" : "i8_mfma_256x256x128_kn_dequant")
-                        : (b_nk ? "i8_mfma_256x256x128_nk" : "i8_mfma_256x256x128_kn");
+  ctx->last_kernel = dq ? (b_nk ? "i8_mfma_256x256x64_ring4_nk_dequant" : "i8_mfma_256x256x64_ring4_kn_dequant")
+                        : (b_nk ? "i8_mfma_256x256x64_ring4_nk" : "i8_mfma_256x256x64_ring4_kn");
   return true;
 }
 

@@ -1,9 +1,11 @@
 // The LDS-tiled MFMA GEMM kernel shared by the bf16, fp16 and int8 families.
 //
-// Workgroup = 256 lanes = 4 waves (2 x 2); macro tile 256 (m) x 256 (n) x 128 BYTES of k
-// (64 halves or 128 int8).  Each wave owns a 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32
-// = 256 accumulators per lane (the AGPR file); one wave per SIMD.  Both operand tiles are
-// 32 KiB; two stages are kept in LDS (128 of the 160 KiB).
+// Workgroup = 256 lanes = 4 waves (2 x 2); macro tile 256 (m) x 256 (n); k is consumed in
+// stages of 64 BYTES per row (32 halves or 64 int8) = two MFMA k-steps.  Each wave owns a
+// 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulators per lane (the AGPR file);
+// one wave per SIMD.  Both operand tiles of a stage are 16 KiB; NSTAGES (4 or 5) stages form
+// a ring in LDS (128 or 160 KiB), NSTAGES-1 of them in flight ahead of the one being
+// multiplied: HBM/L2 latency here is of the order of a microsecond, two to three stage times.
 //
 // Global -> LDS goes straight through the LDS-DMA path (global_load_lds_dwordx4): no
 // staging registers, no ds_write.  One such instruction deposits the wave's 64 x 16 bytes
@@ -11,23 +13,26 @@
 // bank-conflict swizzle is therefore applied on the global side (the chunk a lane fetches),
 // and LDS slot s of a row holds chunk s ^ swizzle(row).
 //
-// A tile  [256 m][128 B of k], as in memory.  16-byte chunk c of row r lives at
-//         r*128 + ((c ^ fA(r)) << 4): the 16-byte fragment reads of 32 consecutive rows
+// A tile  [256 m][64 B of k], as in memory.  16-byte chunk c of row r lives at
+//         r*64 + ((c ^ fA(r)) << 4): the 16-byte fragment reads of 32 consecutive rows
 //         then spread over all banks.
 // B tile  one of
-//   NK    [256 n][128 B of k]  (weights, k contiguous): same geometry and reads as A;
-//   KN16  [64 k][256 n] halves, KN8 [128 k][256 n] bytes (n contiguous, as C = A.B stores
+//   NK    [256 n][64 B of k]  (weights, k contiguous): same geometry and reads as A;
+//   KN16  [32 k][256 n] halves, KN8 [64 k][256 n] bytes (n contiguous, as C = A.B stores
 //         B).  The MFMA wants k contiguous per lane, so fragments come from the transposing
 //         LDS reads ds_read_b64_tr_b16 / _tr_b8: within 16 lanes, lane i supplies the
 //         address of 8 bytes of row k0 + i/4 (i/2 for bytes) and receives the 4 (8)
 //         k-values of column n0 + i.  Chunks are XOR-swizzled by k so that the rows one
 //         instruction touches fall in different banks.
 //
-// Pipeline (per 128-byte k stage = 4 MFMA k-steps of 16 MFMAs each): fragments are double
-// buffered in registers, the reads of k-step s+1 are issued under the MFMAs of k-step s.
-// After k-step 2 the wave waits for its DMA of the next stage, crosses the single barrier
-// of the iteration, issues the DMA of the stage after next into the buffer just drained,
-// and reads the first fragments of the next stage under the MFMAs of k-step 3.
+// Pipeline, iteration s (stage s sits in ring slot s % NSTAGES):
+//   k-step 0: 16 MFMAs on the fragments of (s,0); under them the 12 LDS reads of (s,1)
+//   wait until this wave's DMA of stage s+1 has landed (vmcnt), workgroup barrier
+//   k-step 1: 16 MFMAs on (s,1); under them the 12 LDS reads of (s+1,0) and the 8 DMA
+//             instructions of stage s+NSTAGES-1, into the slot stage s-1 just left (every
+//             wave finished reading it before it reached the barrier).
+// Fragments are double buffered in registers.  The emitted order is pinned slot by slot
+// with scheduling fences: one MFMA, at most one LDS read, at most one DMA.
 //
 // The MFMA is issued with the B fragment as its first operand and the A fragment as its
 // second, so it yields the transposed 32 x 32 block: lane l holds, for the single output
@@ -43,18 +48,20 @@ namespace cig {
 namespace tile {
 
 constexpr int BM = 256, BN = 256;
-constexpr int KB = 128;                    // bytes of k per stage, per row
-constexpr int OPERAND_BYTES = 256 * KB;    // 32 KiB, either operand
+constexpr int KB = 64;                     // bytes of k per stage, per row
+constexpr int OPERAND_BYTES = 256 * KB;    // 16 KiB, either operand
 constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
-constexpr int LDS_BYTES = 2 * STAGE_BYTES;  // 128 KiB of the 160 KiB
+constexpr int DMA_PER_STAGE = 8;           // per wave: 4 A + 4 B instructions of 1 KiB
 
 typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) void global_void;
 
-// ---- A-like tile: [256 rows][8 chunks] ----------------------------------------------------
-__device__ __forceinline__ int rowmajor_swz(int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); }
+// ---- A-like tile: [256 rows][4 chunks] ----------------------------------------------------
+__device__ __forceinline__ int rowmajor_swz(int r) {
+  return ((r >> 2) & 1) | ((((r >> 1) ^ (r >> 3)) & 1) << 1);
+}
 __device__ __forceinline__ int rowmajor_off(int r, int c) {
   return r * KB + ((c ^ rowmajor_swz(r)) << 4);
 }
@@ -64,16 +71,16 @@ enum BMode { B_NK = 0, B_KN16 = 1, B_KN8 = 2 };
 template <int MODE>
 struct BTile;
 
-// DMA geometry of a tile: wave w issues instruction i (0..7); the instruction fills 1 KiB of
+// DMA geometry of a tile: wave w issues instruction i (0..3); the instruction fills 1 KiB of
 // LDS starting at dma_lds(w, i); lane l fetches the 16 bytes at global byte offset
 // dma_src(w, i, l, ld) from the tile's origin (row stride ld bytes).
 
-// [256 rows][128 B]: one instruction = 8 rows.
+// [256 rows][64 B]: one instruction = 16 rows.
 struct RowMajorDma {
-  static __device__ __forceinline__ int dma_lds(int w, int i) { return (64 * w + 8 * i) * KB; }
+  static __device__ __forceinline__ int dma_lds(int w, int i) { return (64 * w + 16 * i) * KB; }
   static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
-    const int r = 64 * w + 8 * i + (l >> 3);
-    return (int64_t)r * ld + (((l & 7) ^ rowmajor_swz(r)) << 4);
+    const int r = 64 * w + 16 * i + (l >> 2);
+    return (int64_t)r * ld + (((l & 3) ^ rowmajor_swz(r)) << 4);
   }
 };
 
@@ -88,7 +95,7 @@ struct BTile<B_NK> : RowMajorDma {
   }
 };
 
-// K x N halves: [64 k][32 chunks of 8 halves]; one DMA instruction = 2 k-rows.
+// K x N halves: [32 k][32 chunks of 8 halves]; one DMA instruction = 2 k-rows.
 template <>
 struct BTile<B_KN16> {
   static __device__ __forceinline__ int swz(int k) {
@@ -96,9 +103,9 @@ struct BTile<B_KN16> {
     return (k3 << 2) | ((((k3 >> 1) ^ k3) & 1) << 1);
   }
   static __device__ __forceinline__ int off(int k, int c) { return k * 512 + ((c ^ swz(k)) << 4); }
-  static __device__ __forceinline__ int dma_lds(int w, int i) { return (16 * w + 2 * i) * 512; }
+  static __device__ __forceinline__ int dma_lds(int w, int i) { return (8 * w + 2 * i) * 512; }
   static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
-    const int k = 16 * w + 2 * i + (l >> 5);
+    const int k = 8 * w + 2 * i + (l >> 5);
     return (int64_t)k * ld + (((l & 31) ^ swz(k)) << 4);
   }
   static __device__ __forceinline__ u32x2 frag_half(const char* sb, int wn, int j, int kk, int h,
@@ -111,16 +118,16 @@ struct BTile<B_KN16> {
   }
 };
 
-// K x N bytes: [128 k][16 chunks of 16 bytes]; one DMA instruction = 4 k-rows.
+// K x N bytes: [64 k][16 chunks of 16 bytes]; one DMA instruction = 4 k-rows.
 template <>
 struct BTile<B_KN8> {
   static __device__ __forceinline__ int swz(int k) {
     return ((k & 7) << 1) | (((k >> 2) ^ (k >> 4)) & 1);
   }
   static __device__ __forceinline__ int off(int k, int c) { return k * 256 + ((c ^ swz(k)) << 4); }
-  static __device__ __forceinline__ int dma_lds(int w, int i) { return (32 * w + 4 * i) * 256; }
+  static __device__ __forceinline__ int dma_lds(int w, int i) { return (16 * w + 4 * i) * 256; }
   static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
-    const int k = 32 * w + 4 * i + (l >> 4);
+    const int k = 16 * w + 4 * i + (l >> 4);
     return (int64_t)k * ld + (((l & 15) ^ swz(k)) << 4);
   }
   static __device__ __forceinline__ u32x2 frag_half(const char* sb, int wn, int j, int kk, int h,
@@ -187,15 +194,17 @@ __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int&
 // four consecutive columns col..col+3 of one output row.
 //
 // A, B are byte pointers; lda/ldb are in BYTES.  K_bytes = K * ELEM_BYTES is a multiple of
-// 128, M and N multiples of 256, all rows 16-byte aligned (the launcher checks).
-template <typename Math, int BMODE, typename Epi>
-__global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tiles_n, int KT,
+// 64, M and N multiples of 256, all rows 16-byte aligned (the launcher checks).  KTS = number
+// of 64-byte stages.
+template <typename Math, int BMODE, int NSTAGES, typename Epi>
+__global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tiles_n, int KTS,
                                                            const char* __restrict__ A,
                                                            int64_t lda,
                                                            const char* __restrict__ B,
                                                            int64_t ldb, Epi epi) {
   typedef typename Math::acc_t acc_t;
   typedef BTile<BMODE> BT;
+  constexpr int DIST = NSTAGES - 1;  // stages in flight ahead of the one being multiplied
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int t = threadIdx.x;
   const int l = t & 63;
@@ -206,9 +215,9 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
   tile_of_workgroup(tiles_m, tiles_n, tm, tn);
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
 
-  // ---- DMA sources: uniform tile origin + per-lane 32-bit byte offsets ----------------------
-  const char* a_tile = A + m0 * lda;  // + kt * KB
-  const char* b_tile;                 // + kt * b_kstep
+  // ---- DMA sources: uniform tile origin + per-lane byte offsets ------------------------------
+  const char* a_tile = A + m0 * lda;  // + stage * KB
+  const char* b_tile;                 // + stage * b_kstep
   int64_t b_kstep;
   if (BMODE == B_NK) {
     b_tile = B + n0 * ldb;
@@ -217,9 +226,9 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
     b_tile = B + n0 * Math::ELEM_BYTES;
     b_kstep = (int64_t)(KB / Math::ELEM_BYTES) * ldb;
   }
-  uint32_t a_voff[8], b_voff[8];
+  uint32_t a_voff[4], b_voff[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < 4; ++i) {
     a_voff[i] = (uint32_t)RowMajorDma::dma_src(w, i, l, lda);
     b_voff[i] = (uint32_t)BT::dma_src(w, i, l, ldb);
   }
@@ -236,14 +245,17 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
                  : "s"(lds_dst), "v"(src)
                  : "m0");
   };
-  // DMA instruction d (0..15) of a stage: even d = A piece d/2, odd d = B piece d/2.
-  auto dma_piece = [&](int kt, int buf, int d) {
-    const uint32_t sa = lds_base + buf * STAGE_BYTES;
+  // DMA instruction d (0..7) of stage `st` into ring slot `slot`: even d = A, odd d = B.
+  // Past the last stage the last one is fetched again (into a slot nobody reads any more),
+  // which keeps the number of outstanding instructions, and so the vmcnt waits, uniform.
+  auto dma_piece = [&](int st, int slot, int d) {
+    st = st < KTS ? st : KTS - 1;
+    const uint32_t sa = lds_base + slot * STAGE_BYTES;
     const int i = d >> 1;
     if (d & 1)
-      dma16(b_tile + (int64_t)kt * b_kstep + b_voff[i], sa + OPERAND_BYTES + BT::dma_lds(w, i));
+      dma16(b_tile + (int64_t)st * b_kstep + b_voff[i], sa + OPERAND_BYTES + BT::dma_lds(w, i));
     else
-      dma16(a_tile + (int64_t)kt * KB + a_voff[i], sa + RowMajorDma::dma_lds(w, i));
+      dma16(a_tile + (int64_t)st * KB + a_voff[i], sa + RowMajorDma::dma_lds(w, i));
   };
 
   const int a_frag_row = wm * 128 + (l & 31);
@@ -254,9 +266,10 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
     u32x4 a[4];
     u32x2 b[8];
   };
-  // LDS read r (0..11) of k-step kk of the stage in `buf`: 0..3 = A fragment r, 4..11 = B half.
-  auto read_piece = [&](Frags& f, int buf, int kk, int r) {
-    const char* sa = lds + buf * STAGE_BYTES;
+  // LDS read r (0..11) of k-step kk of the stage in ring slot `slot`: 0..3 = A fragment r,
+  // 4..11 = B half.
+  auto read_piece = [&](Frags& f, int slot, int kk, int r) {
+    const char* sa = lds + slot * STAGE_BYTES;
     if (r < 4)
       f.a[r] = *reinterpret_cast<const u32x4*>(sa + rowmajor_off(a_frag_row + 32 * r, 2 * kk + g));
     else
@@ -281,49 +294,51 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
 
   Frags f0, f1;
 
-  // prologue: stages 0 and 1 in flight, first fragments in registers
+  // s_waitcnt vmcnt(n), everything else unconstrained: vmcnt is split over bits 3:0 and 15:14.
+  auto wait_vmcnt = [](auto n_const) {
+    constexpr int n = decltype(n_const)::value;
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+  };
+
+  // prologue: stages 0 .. DIST-1 in flight; stage 0 landed; first fragments in registers
 #pragma unroll
-  for (int d = 0; d < 16; ++d) dma_piece(0, 0, d);
-  if (KT > 1) {
+  for (int st = 0; st < DIST; ++st)
 #pragma unroll
-    for (int d = 0; d < 16; ++d) dma_piece(1, 1, d);
-    __builtin_amdgcn_s_waitcnt(0x4f70);  // vmcnt(16): stage 0 landed, stage 1 may be in flight
-  } else {
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-  }
+    for (int d = 0; d < DMA_PER_STAGE; ++d) dma_piece(st, st, d);
+  wait_vmcnt(std::integral_constant<int, DMA_PER_STAGE*(DIST - 1)>{});
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int r = 0; r < 12; ++r) read_piece(f0, 0, 0, r);
 
-  // One k-step: 16 slots, each one MFMA on `cur` plus at most one LDS read into `nxt` (the
-  // operands of the following k-step) and at most one DMA instruction; the fences keep the
-  // emitted order equal to this one.
-#define CIG_KSTEP(cur, nxt, rbuf, rkk, WITH_DMA, dkt, dbuf)          \
-  _Pragma("unroll") for (int sl = 0; sl < 16; ++sl) {                \
-    mfma_piece(cur, sl);                                             \
-    if (sl < 12) read_piece(nxt, rbuf, rkk, sl);                     \
-    if (WITH_DMA) dma_piece(dkt, dbuf, sl);                          \
-    __builtin_amdgcn_sched_barrier(0);                               \
-  }
-
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    CIG_KSTEP(f0, f1, buf, 1, false, 0, 0);  // MFMA (kt,0), read (kt,1)
-    CIG_KSTEP(f1, f0, buf, 2, false, 0, 0);  // MFMA (kt,1), read (kt,2)
-    CIG_KSTEP(f0, f1, buf, 3, false, 0, 0);  // MFMA (kt,2), read (kt,3)
-    // stage kt fully read by this wave; stage kt+1 must have landed for everybody
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+  // Ring slots of the stage being multiplied, of the next one, and of the one the DMA fills
+  // (wave-uniform scalars, advanced modulo NSTAGES each iteration).
+  int slot = 0, next_slot = 1, dma_slot = DIST;
+  for (int s = 0; s < KTS; ++s) {
+    // k-step 0
+#pragma unroll
+    for (int sl = 0; sl < 16; ++sl) {
+      mfma_piece(f0, sl);
+      if (sl < 12) read_piece(f1, slot, 1, sl);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // stage s+1 landed for this wave (stages s+2 .. s+DIST-1 may still be in flight)
+    wait_vmcnt(std::integral_constant<int, DMA_PER_STAGE*(DIST - 2)>{});
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    // Branch-free so the iteration stays straight-line code: past the end the last stage is
-    // fetched again into the buffer nobody reads any more, and the fragment reads of the
-    // (non-existent) next stage are harmless LDS reads.
-    const int knext = kt + 2 < KT ? kt + 2 : KT - 1;
-    CIG_KSTEP(f1, f0, buf ^ 1, 0, true, knext, buf);  // MFMA (kt,3), read (kt+1,0), DMA kt+2
+    // k-step 1
+#pragma unroll
+    for (int sl = 0; sl < 16; ++sl) {
+      mfma_piece(f1, sl);
+      if (sl < 12) read_piece(f0, next_slot, 0, sl);
+      if (sl & 1) dma_piece(s + DIST, dma_slot, sl >> 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    slot = next_slot;
+    next_slot = next_slot + 1 == NSTAGES ? 0 : next_slot + 1;
+    dma_slot = dma_slot + 1 == NSTAGES ? 0 : dma_slot + 1;
   }
-#undef CIG_KSTEP
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): no DMA outlives the main loop
+  wait_vmcnt(std::integral_constant<int, 0>{});  // no DMA outlives the main loop
 
   // acc[i][j][4q+e] = C[m0 + wm*128 + 32i + l%32][n0 + wn*128 + 32j + 8q + 4g + e]
 #pragma unroll
@@ -338,10 +353,14 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
   }
 }
 
-template <typename Math, int BMODE, typename Epi>
+constexpr int DEFAULT_STAGES = 4;
+
+template <typename Math, int BMODE, typename Epi, int NSTAGES = DEFAULT_STAGES>
 void launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
                  int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi) {
-  auto kern = mfma_tile_kernel<Math, BMODE, Epi>;
+  static_assert(NSTAGES == 4 || NSTAGES == 5, "ring of 4 or 5 stages");
+  constexpr int LDS_BYTES = NSTAGES * STAGE_BYTES;
+  auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, Epi>;
   static int attr_device = -1;  // one per template instance
   if (attr_device != ctx->device) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
