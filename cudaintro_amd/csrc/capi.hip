@@ -89,6 +89,17 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->stream = nullptr;
   ctx->last_kernel = "";
   ctx->last_error[0] = '\0';
+  ctx->ws_partial_bytes = (size_t)16 << 20;
+  ctx->ws_counter_bytes = (size_t)64 << 10;
+  ctx->workspace = nullptr;
+  if (hipMalloc(&ctx->workspace, ctx->ws_partial_bytes + ctx->ws_counter_bytes) != hipSuccess ||
+      hipMemset(static_cast<char*>(ctx->workspace) + ctx->ws_partial_bytes, 0,
+                ctx->ws_counter_bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    if (ctx->workspace) (void)hipFree(ctx->workspace);
+    delete ctx;
+    return CIGEMM_STATUS_ALLOC_FAILED;
+  }
   *handle = ctx;
   return CIGEMM_STATUS_SUCCESS;
 }
@@ -96,6 +107,7 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
 cigemmStatus_t cigemmDestroy(cigemmHandle_t h) {
   if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
   h->magic = 0;
+  if (h->workspace) (void)hipFree(h->workspace);
   delete h;
   return CIGEMM_STATUS_SUCCESS;
 }

@@ -16,6 +16,11 @@ struct cigemmContext {
   int num_cus;
   hipStream_t stream;
   const char* last_kernel;
+  // Device scratch of the split-K kernels, allocated once at create: `ws_partial_bytes` of
+  // partial sums followed by `ws_counter_bytes` of arrival counters (zero between calls).
+  void* workspace;
+  size_t ws_partial_bytes;
+  size_t ws_counter_bytes;
   char last_error[256];
 };
 

@@ -2,26 +2,10 @@
 // in, fp32 accumulate (v_mfma_f32_32x32x16_{f16,bf16}), one round-to-nearest-even narrowing
 // out.  The kernel itself is the shared LDS-tiled MFMA kernel; this file supplies the
 // 16-bit epilogue and the shape gate.
+#include "epilogues.h"
 #include "mfma_tile.h"
 
 namespace cig {
-namespace {
-
-// Narrows four consecutive columns and stores them as one 8-byte piece.
-template <typename E16>
-struct EpiStore16x4 {
-  uint16_t* C;
-  int64_t ldc;
-  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float v0, float v1, float v2,
-                                             float v3) const {
-    u32x2 v;
-    v[0] = (uint32_t)E16::narrow(v0) | ((uint32_t)E16::narrow(v1) << 16);
-    v[1] = (uint32_t)E16::narrow(v2) | ((uint32_t)E16::narrow(v3) << 16);
-    *reinterpret_cast<u32x2*>(C + r * ldc + c) = v;
-  }
-};
-
-}  // namespace
 
 bool launch_16b_mfma(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_t K,
                      const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, uint16_t* C,

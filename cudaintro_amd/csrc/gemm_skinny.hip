@@ -1,8 +1,371 @@
-// Skinny (decode-shape) GEMM placeholder gate.
-#include "common.h"
+// Skinny (decode-shape) GEMMs: y[M x N] = x[M x K] . W with M <= 32.  The weights are read
+// once and nothing is reused, so these kernels are bound by HBM bandwidth; they exist to keep
+// a deep, wide stream of weight bytes in flight, not to save arithmetic.
+//
+// Workgroup = 256 lanes = 4 waves; it owns BN output columns and one K range (split-K), and
+// walks its K range in stages held in a ring in LDS (7 or 8 stages, 140-144 KiB): one stage =
+// one weight tile (16 KiB) + the matching slice of x, all moved by LDS-DMA, NSTAGES-1 stages
+// in flight.  The arithmetic is the 32x32 MFMA with x padded to 32 rows (rows >= M re-read
+// row M-1 and are never stored): at M <= 32 the matrix core is idle most of the time anyway.
+//
+//   16-bit, W is K x N (n contiguous):  BN = 256, stage = 32 k: W tile [32 k][256 n] read back
+//       with the transposing LDS read (same layout as the big tile kernel), x tile [32 m][64 B].
+//   int8, W is N x K (k contiguous):    BN = 128, stage = 128 k: W tile [128 n][128 B],
+//       x tile [32 m][128 B], both read with 16-byte LDS reads.
+//
+// Split-K: each workgroup writes its 32 x BN partial (fp32 / int32) to the handle's
+// workspace, then bumps a per-column-slab counter; the workgroup that finds it is the last
+// one sums the partials in split order (so the result does not depend on arrival order),
+// applies the epilogue and resets the counter.
+#include "epilogues.h"
+#include "mfma_tile.h"
+
 namespace cig {
-bool launch_skinny_16(cigemmContext*, bool, int64_t, int64_t, int64_t, const uint16_t*, int64_t,
-                      const uint16_t*, int64_t, uint16_t*, int64_t) { return false; }
-bool launch_skinny_i8(cigemmContext*, int64_t, int64_t, int64_t, const int8_t*, int64_t,
-                      const int8_t*, int64_t, bool, int32_t*, int64_t, const DequantArgs*) { return false; }
+namespace {
+
+using tile::lds_void;
+
+constexpr int XROWS = 32;  // x padded to one MFMA tile of rows
+
+__device__ __forceinline__ void dma16(const char* src, uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_dst), "v"(src)
+               : "m0");
+}
+__device__ __forceinline__ void dma4(const char* src, uint32_t lds_dst) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+               :
+               : "s"(lds_dst), "v"(src)
+               : "m0");
+}
+
+// ---- 16-bit weights, K x N ------------------------------------------------------------------
+template <typename MathT>
+struct GeoKN16 {
+  typedef MathT Math;
+  typedef tile::BTile<tile::B_KN16> WT;
+  static constexpr int BN = 256;
+  static constexpr int K_ELEMS = 32;                 // k per stage
+  static constexpr int W_BYTES = 32 * 512;           // [32 k][256 n] halves
+  static constexpr int X_BYTES = XROWS * 64;         // [32 m][64 B]
+  static constexpr int STAGE_BYTES = W_BYTES + X_BYTES;
+  static constexpr int NSTAGES = 8;                  // 144 KiB
+  static constexpr int DMA_PER_STAGE = 6;            // per wave: 4 W (1 KiB) + 2 x (256 B)
+  static constexpr int NT = 2;                       // 32-column tiles per wave
+
+  // W points at (k = first k of the stage, n = n0); x at (row 0, same k), both in bytes.
+  static __device__ __forceinline__ void dma(const char* W, int64_t ldw, const char* x, int64_t ldx,
+                                             int M, uint32_t slot_lds, int w, int l) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      dma16(W + WT::dma_src(w, i, l, ldw), slot_lds + WT::dma_lds(w, i));
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = 8 * w + 4 * i + (l >> 4);
+      const int rr = r < M ? r : M - 1;
+      const int chunk = ((l & 15) >> 2) ^ tile::rowmajor_swz(r);
+      dma4(x + (int64_t)rr * ldx + (chunk << 4) + ((l & 3) << 2),
+           slot_lds + W_BYTES + (8 * w + 4 * i) * 64);
+    }
+  }
+  static __device__ __forceinline__ void compute(const char* slot, int w, int l,
+                                                 typename Math::acc_t (&acc)[NT]) {
+    const char* sx = slot + W_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const u32x4 xf =
+          *reinterpret_cast<const u32x4*>(sx + tile::rowmajor_off(l & 31, 2 * kk + (l >> 5)));
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const u32x2 lo = WT::frag_half(slot, 0, 2 * w + j, kk, 0, l);
+        const u32x2 hi = WT::frag_half(slot, 0, 2 * w + j, kk, 1, l);
+        acc[j] = Math::mfma(__builtin_shufflevector(lo, hi, 0, 1, 2, 3), xf, acc[j]);
+      }
+    }
+  }
+  // first column (relative to n0) of accumulator quad q of tile j
+  static __device__ __forceinline__ int col(int w, int j, int q, int l) {
+    return 64 * w + 32 * j + 8 * q + 4 * (l >> 5);
+  }
+  static __device__ __forceinline__ int64_t w_stage_step(int64_t ldw) { return 32 * ldw; }
+  static constexpr int X_STAGE_STEP = 64;
+};
+
+// ---- int8 weights, N x K ----------------------------------------------------------------------
+struct GeoNK8 {
+  typedef tile::MathI8 Math;
+  static constexpr int BN = 128;
+  static constexpr int K_ELEMS = 128;
+  static constexpr int W_BYTES = 128 * 128;          // [128 n][128 B]
+  static constexpr int X_BYTES = XROWS * 128;        // [32 m][128 B]
+  static constexpr int STAGE_BYTES = W_BYTES + X_BYTES;
+  static constexpr int NSTAGES = 7;                  // 140 KiB
+  static constexpr int DMA_PER_STAGE = 5;            // per wave: 4 W + 1 x, 1 KiB each
+  static constexpr int NT = 1;
+
+  // 128-byte rows, 8 chunks: chunk c of row r at r*128 + ((c ^ swz(r)) << 4)
+  static __device__ __forceinline__ int swz(int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); }
+  static __device__ __forceinline__ int off(int r, int c) { return r * 128 + ((c ^ swz(r)) << 4); }
+
+  static __device__ __forceinline__ void dma(const char* W, int64_t ldw, const char* x, int64_t ldx,
+                                             int M, uint32_t slot_lds, int w, int l) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 32 * w + 8 * i + (l >> 3);
+      dma16(W + (int64_t)r * ldw + (((l & 7) ^ swz(r)) << 4), slot_lds + (32 * w + 8 * i) * 128);
+    }
+    const int r = 8 * w + (l >> 3);
+    const int rr = r < M ? r : M - 1;
+    dma16(x + (int64_t)rr * ldx + (((l & 7) ^ swz(r)) << 4), slot_lds + W_BYTES + (8 * w) * 128);
+  }
+  static __device__ __forceinline__ void compute(const char* slot, int w, int l,
+                                                 Math::acc_t (&acc)[NT]) {
+    const char* sx = slot + W_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const u32x4 xf = *reinterpret_cast<const u32x4*>(sx + off(l & 31, 2 * kk + (l >> 5)));
+      const u32x4 wf =
+          *reinterpret_cast<const u32x4*>(slot + off(32 * w + (l & 31), 2 * kk + (l >> 5)));
+      acc[0] = Math::mfma(wf, xf, acc[0]);
+    }
+  }
+  static __device__ __forceinline__ int col(int w, int j, int q, int l) {
+    return 32 * w + 8 * q + 4 * (l >> 5);
+  }
+  static __device__ __forceinline__ int64_t w_stage_step(int64_t) { return 128; }
+  static constexpr int X_STAGE_STEP = 128;
+};
+
+template <typename Geo>
+__device__ __forceinline__ const char* w_origin(const char* W, int64_t ldw, int64_t n0,
+                                                int64_t k0_elems);
+template <>
+__device__ __forceinline__ const char* w_origin<GeoNK8>(const char* W, int64_t ldw, int64_t n0,
+                                                        int64_t k0) {
+  return W + n0 * ldw + k0;
+}
+template <typename Geo>
+__device__ __forceinline__ const char* w_origin(const char* W, int64_t ldw, int64_t n0,
+                                                int64_t k0) {
+  return W + k0 * ldw + n0 * 2;  // K x N halves
+}
+
+// Four partial sums as raw 32-bit words, one 16-byte store.
+template <typename T>
+__device__ __forceinline__ void store_partial(uint32_t* dst, T v0, T v1, T v2, T v3) {
+  u32x4 v = {__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
+             __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)};
+  *reinterpret_cast<u32x4*>(dst) = v;
+}
+
+// Workspace layout: partials[split][32][N] (4-byte words) followed by one counter per slab.
+template <typename Geo, typename Epi>
+__global__ __launch_bounds__(256, 1) void skinny_kernel(int M, int N, int stages_per_split,
+                                                        int splits, const char* __restrict__ X,
+                                                        int64_t ldx, const char* __restrict__ W,
+                                                        int64_t ldw, Epi epi,
+                                                        uint32_t* __restrict__ partials,
+                                                        uint32_t* __restrict__ counters) {
+  typedef typename Geo::Math Math;
+  typedef typename Math::acc_t acc_t;
+  typedef typename Math::scalar_t scalar_t;
+  constexpr int NS = Geo::NSTAGES, DIST = NS - 1, DPS = Geo::DMA_PER_STAGE;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  __shared__ int is_last;
+  const int t = threadIdx.x, l = t & 63;
+  const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int slab = blockIdx.x / splits, split = blockIdx.x % splits;
+  const int64_t n0 = (int64_t)slab * Geo::BN;
+  const int64_t k0 = (int64_t)split * stages_per_split * Geo::K_ELEMS;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+
+  const char* w_src = w_origin<Geo>(W, ldw, n0, k0);
+  const char* x_src = X + k0 * Math::ELEM_BYTES;
+  const int64_t w_step = Geo::w_stage_step(ldw);
+  const int KTS = stages_per_split;
+
+  auto issue = [&](int st, int slot) {
+    st = st < KTS ? st : KTS - 1;  // past the end: refetch the last stage into a dead slot
+    Geo::dma(w_src + st * w_step, ldw, x_src + (int64_t)st * Geo::X_STAGE_STEP, ldx, M,
+             lds_base + slot * Geo::STAGE_BYTES, w, l);
+  };
+  auto wait_vmcnt = [](auto n_const) {
+    constexpr int n = decltype(n_const)::value;
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+  };
+
+  acc_t acc[Geo::NT];
+#pragma unroll
+  for (int j = 0; j < Geo::NT; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[j][e] = 0;
+
+#pragma unroll
+  for (int st = 0; st < DIST; ++st) issue(st, st);
+
+  int slot = 0, dma_slot = DIST;
+  for (int s = 0; s < KTS; ++s) {
+    // stage s landed for this wave (stages s+1 .. s+DIST-1 may be in flight); after the barrier
+    // it is visible to all waves and every wave has finished reading stage s-1
+    wait_vmcnt(std::integral_constant<int, DPS*(DIST - 1)>{});
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    issue(s + DIST, dma_slot);
+    Geo::compute(lds + slot * Geo::STAGE_BYTES, w, l, acc);
+    slot = slot + 1 == NS ? 0 : slot + 1;
+    dma_slot = dma_slot + 1 == NS ? 0 : dma_slot + 1;
+  }
+  wait_vmcnt(std::integral_constant<int, 0>{});
+
+  const int m = l & 31;
+  if (splits == 1) {
+    if (m < M) {
+#pragma unroll
+      for (int j = 0; j < Geo::NT; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          epi(m, n0 + Geo::col(w, j, q, l), acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2],
+              acc[j][4 * q + 3]);
+    }
+    return;
+  }
+
+  // ---- split-K: publish the partial, last workgroup of the slab reduces in split order -------
+  if (m < M) {
+#pragma unroll
+    for (int j = 0; j < Geo::NT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        store_partial(partials + ((int64_t)split * XROWS + m) * N + n0 + Geo::col(w, j, q, l),
+                      acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]);
+  }
+  __threadfence();
+  __syncthreads();
+  if (t == 0) {
+    const uint32_t old = __hip_atomic_fetch_add(counters + slab, 1u, __ATOMIC_ACQ_REL,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+    is_last = old == (uint32_t)(splits - 1);
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+  if (m < M) {
+#pragma unroll
+    for (int j = 0; j < Geo::NT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        scalar_t sum[4] = {0, 0, 0, 0};
+        const int64_t at = (int64_t)m * N + n0 + Geo::col(w, j, q, l);
+        for (int sp = 0; sp < splits; ++sp) {
+          const uint32_t* p = partials + (int64_t)sp * XROWS * N + at;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            sum[e] += __builtin_bit_cast(
+                scalar_t, __hip_atomic_load(p + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        }
+        epi(m, n0 + Geo::col(w, j, q, l), sum[0], sum[1], sum[2], sum[3]);
+      }
+  }
+  if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Number of K splits: enough workgroups to cover the chip about once, at least 4 stages per
+// split, and partials that fit the workspace.
+template <typename Geo>
+int choose_splits(const cigemmContext* ctx, int64_t N, int64_t kts) {
+  const int64_t slabs = N / Geo::BN;
+  int64_t s = (ctx->num_cus + slabs - 1) / slabs;
+  if (s > 16) s = 16;
+  while (s > 1 && (kts % s || kts / s < 4)) --s;
+  while (s > 1 && (size_t)s * XROWS * N * 4 > ctx->ws_partial_bytes) --s;
+  if (s > 1 && kts % s) s = 1;
+  if ((size_t)slabs * 4 > ctx->ws_counter_bytes) s = 1;
+  return (int)(s < 1 ? 1 : s);
+}
+
+template <typename Geo, typename Epi>
+void launch_skinny(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
+                   int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
+  constexpr int LDS_BYTES = Geo::NSTAGES * Geo::STAGE_BYTES;
+  auto kern = skinny_kernel<Geo, Epi>;
+  static int attr_device = -1;
+  if (attr_device != ctx->device) {
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              LDS_BYTES);
+    attr_device = ctx->device;
+  }
+  const int64_t kts = K / Geo::K_ELEMS;
+  const int splits = choose_splits<Geo>(ctx, N, kts);
+  const unsigned grid = (unsigned)((N / Geo::BN) * splits);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS_BYTES, ctx->stream, (int)M, (int)N,
+                     (int)(kts / splits), splits, static_cast<const char*>(X), ldx_bytes,
+                     static_cast<const char*>(W), ldw_bytes, epi,
+                     static_cast<uint32_t*>(ctx->workspace),
+                     reinterpret_cast<uint32_t*>(static_cast<char*>(ctx->workspace) +
+                                                 ctx->ws_partial_bytes));
+}
+
+template <typename Geo>
+bool skinny_shape_ok(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K, int elem,
+                     const void* X, int64_t ldx, const void* W, int64_t ldw) {
+  if (!ctx->workspace) return false;
+  if (M < 1 || M > XROWS || N <= 0 || K <= 0) return false;
+  if (N % Geo::BN || K % Geo::K_ELEMS) return false;
+  if ((ldx * elem) % 16 || (ldw * elem) % 16) return false;
+  if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return false;
+  if (N / Geo::BN * 16 > 2147483647LL || N > 2147483647LL) return false;
+  return true;
+}
+
+}  // namespace
+
+bool launch_skinny_16(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_t K,
+                      const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, uint16_t* C,
+                      int64_t ldc) {
+  typedef GeoKN16<tile::MathBF16> GB;
+  typedef GeoKN16<tile::MathF16> GF;
+  if (!skinny_shape_ok<GB>(ctx, M, N, K, 2, A, lda, B, ldb)) return false;
+  if (ldc % 4 || ((uintptr_t)C & 7)) return false;
+  if (bf16) {
+    launch_skinny<GB>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<BF16>{C, ldc});
+    ctx->last_kernel = "bf16_skinny_32x256_ring8";
+  } else {
+    launch_skinny<GF>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<F16>{C, ldc});
+    ctx->last_kernel = "f16_skinny_32x256_ring8";
+  }
+  return true;
+}
+
+bool launch_skinny_i8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                      int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
+                      int64_t ldc, const DequantArgs* dq) {
+  if (!b_nk) return false;  // K x N int8 weights at M <= 32 go to the any-shape kernel
+  if (!skinny_shape_ok<GeoNK8>(ctx, M, N, K, 1, A, lda, B, ldb)) return false;
+  if (!dq) {
+    if (ldc % 4 || ((uintptr_t)C & 15)) return false;
+    launch_skinny<GeoNK8>(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32x4{C, ldc});
+    ctx->last_kernel = "i8_skinny_32x128_ring7_nk";
+    return true;
+  }
+  if (dq->out_bf16 ? (dq->ldo % 4 || ((uintptr_t)dq->out & 7))
+                   : (dq->ldo % 4 || ((uintptr_t)dq->out & 15)))
+    return false;
+  if (dq->sb_vec && ((uintptr_t)dq->sb & 15)) return false;
+  if (dq->acc_out && (dq->ldacc % 4 || ((uintptr_t)dq->acc_out & 15))) return false;
+#define CIG_DQ(OB, DA)                                                                          \
+  launch_skinny<GeoNK8>(ctx, M, N, K, A, lda, B, ldb,                                           \
+                        EpiDequantX4<OB, DA>{dq->out, dq->ldo, dq->sa, dq->sb, dq->sa_vec,      \
+                                             dq->sb_vec, dq->acc_out, dq->ldacc})
+  const bool dump = dq->acc_out != nullptr;
+  if (dq->out_bf16) {
+    if (dump) CIG_DQ(true, true); else CIG_DQ(true, false);
+  } else {
+    if (dump) CIG_DQ(false, true); else CIG_DQ(false, false);
+  }
+#undef CIG_DQ
+  ctx->last_kernel = "i8_skinny_32x128_ring7_nk_dequant";
+  return true;
+}
+
 }  // namespace cig

@@ -1,0 +1,117 @@
+"""Skinny (decode-shape) GEMMs, M <= 32, through the C ABI: the split-K kernels against the
+oracle.  int8 accumulators and dequantized outputs bit-exact; 16-bit within the K-scaled bound
+and bit-exact on exact-arithmetic inputs; repeated calls (the arrival counters must return to
+zero) give identical results."""
+import numpy as np
+import pytest
+
+import cudaintro_amd as ci
+from cudaintro_amd import workloads as wl
+from gpu_util import bits, error_bound_16, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def widen(oracle, b, kind):
+    return oracle.bf16_to_f32(b) if kind == "bf16" else oracle.f16_to_f32(b)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("M", [1, 2, 8, 17, 32])
+@pytest.mark.parametrize("N,K", [(256, 128), (512, 1024), (8192, 8192), (2048, 4096 + 32)])
+def test_skinny_16bit(handle, torch_gpu, oracle, kind, M, N, K):
+    torch = torch_gpu
+    xb, wb = wl.normal_16bit(M, N, K, seed=4, kind=kind, sigma_b=0.02)
+    x, w = to_dev(torch, xb, kind), to_dev(torch, wb, kind)
+    fn = handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16
+    y = fn(x, w)
+    assert "skinny" in handle.last_kernel, handle.last_kernel
+    ref, S = oracle.gemm_f64(widen(oracle, xb, kind), widen(oracle, wb, kind), with_abs=True)
+    got = widen(oracle, bits(torch, y), kind).astype(np.float64)
+    err = np.abs(got - ref)
+    bound = error_bound_16(ref, S, K, kind)
+    assert (err <= bound).all(), float((err / bound).max())
+    # a second and third call reuse the workspace and counters
+    for _ in range(2):
+        assert torch.equal(fn(x, w), y)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+def test_skinny_16bit_exact_inputs(handle, torch_gpu, oracle, rng, kind):
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    narrow = oracle.f32_to_bf16 if kind == "bf16" else oracle.f32_to_f16
+    for (M, N, K) in [(1, 256, 64), (5, 1024, 2048), (32, 8192, 1024)]:
+        X = rng.choice(vals, size=(M, K))
+        W = rng.choice(vals, size=(K, N))
+        fn = handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16
+        y = fn(to_dev(torch_gpu, narrow(X), kind), to_dev(torch_gpu, narrow(W), kind))
+        assert "skinny" in handle.last_kernel
+        np.testing.assert_array_equal(bits(torch_gpu, y), narrow(oracle.gemm_f32(X, W)))
+
+
+@pytest.mark.parametrize("kind", ["bf16"])
+def test_skinny_onehot_and_padding_rows(handle, torch_gpu, oracle, rng, kind):
+    """Row m of x one-hot at k_m selects row k_m of W; rows >= M of the padded tile are never
+    stored (the output buffer has guard rows)."""
+    torch = torch_gpu
+    M, N, K = 7, 512, 256
+    Wf = oracle.bf16_to_f32(oracle.f32_to_bf16(rng.normal(size=(K, N)).astype(np.float32)))
+    ks = rng.integers(0, K, size=M)
+    X = np.zeros((M, K), np.float32)
+    X[np.arange(M), ks] = 1.0
+    out = torch.full((M + 4, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    handle.gemm_bf16(to_dev(torch, oracle.f32_to_bf16(X), kind), to_dev(torch, oracle.f32_to_bf16(Wf), kind),
+                     out=out[:M])
+    assert "skinny" in handle.last_kernel
+    o = bits(torch, out)
+    np.testing.assert_array_equal(o[:M], oracle.f32_to_bf16(Wf[ks]))
+    assert (o[M:] == oracle.f32_to_bf16(np.float32(7.0))).all()
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 32])
+@pytest.mark.parametrize("N,K", [(128, 128), (1024, 512), (8192, 8192), (384, 4096 + 128)])
+@pytest.mark.parametrize("out_type", ["i32", "f32", "bf16"])
+def test_skinny_int8_nk(handle, torch_gpu, oracle, rng, M, N, K, out_type):
+    torch = torch_gpu
+    X = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    acc_ref = oracle.gemm_i8_i32(X, W, b_is_nk=True)
+    xd, wd = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda()
+    if out_type == "i32":
+        for _ in range(2):
+            y = handle.gemm_i8_i32(xd, wd, ci.B_NK)
+            assert "skinny" in handle.last_kernel, handle.last_kernel
+            np.testing.assert_array_equal(y.cpu().numpy(), acc_ref)
+        return
+    sa = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
+    sb = rng.uniform(1e-3, 5e-2, N).astype(np.float32)
+    ot = ci.OUT_BF16 if out_type == "bf16" else ci.OUT_F32
+    out, acc = handle.gemm_i8_dequant(xd, wd, torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda(),
+                                      ci.B_NK, ot, dump_acc=True)
+    assert "skinny" in handle.last_kernel, handle.last_kernel
+    np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
+    expect = oracle.dequant(acc_ref, sa, sb, out_dtype=out_type, sa_per_row=M > 1, sb_per_col=True)
+    got = bits(torch, out) if out_type == "bf16" else out.cpu().numpy()
+    np.testing.assert_array_equal(got, expect)
+
+
+def test_config_skinny_decode(handle, torch_gpu, oracle):
+    """The decode-shaped configurations: M in {1, 8, 32}, N = K = 8192, bf16 weights N(0,0.02)
+    and int8 weights with per-channel scales."""
+    torch = torch_gpu
+    for M in (1, 8, 32):
+        xb, wb = wl.skinny_bf16(M, 8192, 8192, seed=4)
+        y = handle.gemm_bf16(to_dev(torch, xb, "bf16"), to_dev(torch, wb, "bf16"))
+        assert "skinny" in handle.last_kernel
+        ref, S = oracle.gemm_f64(oracle.bf16_to_f32(xb), oracle.bf16_to_f32(wb), with_abs=True)
+        got = oracle.bf16_to_f32(bits(torch, y)).astype(np.float64)
+        assert (np.abs(got - ref) <= error_bound_16(ref, S, 8192, "bf16")).all()
+        xq, sx, wq, sw = wl.skinny_int8(M, 8192, 8192, seed=4)
+        out, acc = handle.gemm_i8_dequant(torch.from_numpy(xq).cuda(), torch.from_numpy(wq).cuda(),
+                                          torch.from_numpy(sx).cuda(), torch.from_numpy(sw).cuda(),
+                                          ci.B_NK, ci.OUT_BF16, dump_acc=True)
+        assert "skinny" in handle.last_kernel
+        acc_ref = oracle.gemm_i8_i32(xq, wq, b_is_nk=True)
+        np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
+        np.testing.assert_array_equal(bits(torch, out),
+                                      oracle.dequant(acc_ref, sx, sw, out_dtype="bf16", sa_per_row=M > 1))
