@@ -151,21 +151,38 @@ __device__ __forceinline__ const char* w_origin(const char* W, int64_t ldw, int6
   return W + k0 * ldw + n0 * 2;  // K x N halves
 }
 
-// Four partial sums as raw 32-bit words, one 16-byte store.
+// Partials cross workgroups on different XCDs, each with its own L2, so they are written
+// and read with agent-scope accesses (which go through to the coherence point) rather than
+// ordinary cached ones plus an agent-scope fence: that fence writes back and invalidates the
+// whole L2 and costs tens of microseconds per call.  A quad of partial sums travels as two
+// 64-bit words; the layout is private to this kernel and lane-contiguous
+// ([split][slab][quad][half][lane]) so every access instruction moves 512 contiguous bytes.
 template <typename T>
-__device__ __forceinline__ void store_partial(uint32_t* dst, T v0, T v1, T v2, T v3) {
-  u32x4 v = {__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
-             __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)};
-  *reinterpret_cast<u32x4*>(dst) = v;
+__device__ __forceinline__ void store_partial(uint64_t* dst, T v0, T v1, T v2, T v3) {
+  const uint64_t lo = (uint64_t)__builtin_bit_cast(uint32_t, v0) |
+                      ((uint64_t)__builtin_bit_cast(uint32_t, v1) << 32);
+  const uint64_t hi = (uint64_t)__builtin_bit_cast(uint32_t, v2) |
+                      ((uint64_t)__builtin_bit_cast(uint32_t, v3) << 32);
+  __hip_atomic_store(dst, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(dst + 256, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+__device__ __forceinline__ void add_partial(const uint64_t* src, T (&sum)[4]) {
+  const uint64_t lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint64_t hi = __hip_atomic_load(src + 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  sum[0] += __builtin_bit_cast(T, (uint32_t)lo);
+  sum[1] += __builtin_bit_cast(T, (uint32_t)(lo >> 32));
+  sum[2] += __builtin_bit_cast(T, (uint32_t)hi);
+  sum[3] += __builtin_bit_cast(T, (uint32_t)(hi >> 32));
 }
 
-// Workspace layout: partials[split][32][N] (4-byte words) followed by one counter per slab.
-template <typename Geo, typename Epi>
+// Workspace: the partials (see store_partial) followed by one arrival counter per slab.
+template <typename Geo, typename Epi, int SPLITS>
 __global__ __launch_bounds__(256, 1) void skinny_kernel(int M, int N, int stages_per_split,
-                                                        int splits, const char* __restrict__ X,
+                                                        const char* __restrict__ X,
                                                         int64_t ldx, const char* __restrict__ W,
                                                         int64_t ldw, Epi epi,
-                                                        uint32_t* __restrict__ partials,
+                                                        uint64_t* __restrict__ partials,
                                                         uint32_t* __restrict__ counters) {
   typedef typename Geo::Math Math;
   typedef typename Math::acc_t acc_t;
@@ -175,6 +192,7 @@ __global__ __launch_bounds__(256, 1) void skinny_kernel(int M, int N, int stages
   __shared__ int is_last;
   const int t = threadIdx.x, l = t & 63;
   const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+  constexpr int splits = SPLITS;
   const int slab = blockIdx.x / splits, split = blockIdx.x % splits;
   const int64_t n0 = (int64_t)slab * Geo::BN;
   const int64_t k0 = (int64_t)split * stages_per_split * Geo::K_ELEMS;
@@ -232,78 +250,89 @@ __global__ __launch_bounds__(256, 1) void skinny_kernel(int M, int N, int stages
   }
 
   // ---- split-K: publish the partial, last workgroup of the slab reduces in split order -------
+  constexpr int QUADS = Geo::NT * 4;
+  const int slabs = gridDim.x / splits;
+  // 64-bit word index of (split sp, this slab, quad 0, half 0, this lane)
+  auto part = [&](int sp) {
+    return partials + ((int64_t)(sp * slabs + slab) * QUADS * 2) * 256 + t;
+  };
   if (m < M) {
+    uint64_t* dst = part(split);
 #pragma unroll
     for (int j = 0; j < Geo::NT; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q)
-        store_partial(partials + ((int64_t)split * XROWS + m) * N + n0 + Geo::col(w, j, q, l),
-                      acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]);
+        store_partial(dst + (j * 4 + q) * 512, acc[j][4 * q], acc[j][4 * q + 1],
+                      acc[j][4 * q + 2], acc[j][4 * q + 3]);
   }
-  __threadfence();
+  // every lane's partial stores have been acknowledged before the arrival is counted
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
   if (t == 0) {
-    const uint32_t old = __hip_atomic_fetch_add(counters + slab, 1u, __ATOMIC_ACQ_REL,
+    const uint32_t old = __hip_atomic_fetch_add(counters + slab, 1u, __ATOMIC_RELAXED,
                                                 __HIP_MEMORY_SCOPE_AGENT);
     is_last = old == (uint32_t)(splits - 1);
   }
   __syncthreads();
   if (!is_last) return;
-  __threadfence();
   if (m < M) {
 #pragma unroll
     for (int j = 0; j < Geo::NT; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         scalar_t sum[4] = {0, 0, 0, 0};
-        const int64_t at = (int64_t)m * N + n0 + Geo::col(w, j, q, l);
-        for (int sp = 0; sp < splits; ++sp) {
-          const uint32_t* p = partials + (int64_t)sp * XROWS * N + at;
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            sum[e] += __builtin_bit_cast(
-                scalar_t, __hip_atomic_load(p + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        }
+        for (int sp = 0; sp < splits; ++sp) add_partial(part(sp) + (j * 4 + q) * 512, sum);
         epi(m, n0 + Geo::col(w, j, q, l), sum[0], sum[1], sum[2], sum[3]);
       }
   }
   if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Number of K splits: enough workgroups to cover the chip about once, at least 4 stages per
-// split, and partials that fit the workspace.
+// Number of K splits, a power of two up to 16: enough workgroups to cover the chip about
+// once, at least 4 stages per split, and partials that fit the workspace.
 template <typename Geo>
 int choose_splits(const cigemmContext* ctx, int64_t N, int64_t kts) {
   const int64_t slabs = N / Geo::BN;
-  int64_t s = (ctx->num_cus + slabs - 1) / slabs;
-  if (s > 16) s = 16;
-  while (s > 1 && (kts % s || kts / s < 4)) --s;
-  while (s > 1 && (size_t)s * XROWS * N * 4 > ctx->ws_partial_bytes) --s;
-  if (s > 1 && kts % s) s = 1;
+  int s = 1;
+  while (s < 16 && slabs * s < ctx->num_cus && kts % (2 * s) == 0 && kts / (2 * s) >= 4 &&
+         (size_t)(2 * s) * XROWS * N * 4 <= ctx->ws_partial_bytes)
+    s *= 2;
   if ((size_t)slabs * 4 > ctx->ws_counter_bytes) s = 1;
-  return (int)(s < 1 ? 1 : s);
+  return s;
 }
 
-template <typename Geo, typename Epi>
-void launch_skinny(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
-                   int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
+template <typename Geo, typename Epi, int SPLITS>
+void launch_skinny_n(cigemmContext* ctx, int64_t M, int64_t N, int64_t kts, const void* X,
+                     int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
   constexpr int LDS_BYTES = Geo::NSTAGES * Geo::STAGE_BYTES;
-  auto kern = skinny_kernel<Geo, Epi>;
+  auto kern = skinny_kernel<Geo, Epi, SPLITS>;
   static int attr_device = -1;
   if (attr_device != ctx->device) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                               LDS_BYTES);
     attr_device = ctx->device;
   }
-  const int64_t kts = K / Geo::K_ELEMS;
-  const int splits = choose_splits<Geo>(ctx, N, kts);
-  const unsigned grid = (unsigned)((N / Geo::BN) * splits);
+  const unsigned grid = (unsigned)((N / Geo::BN) * SPLITS);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS_BYTES, ctx->stream, (int)M, (int)N,
-                     (int)(kts / splits), splits, static_cast<const char*>(X), ldx_bytes,
+                     (int)(kts / SPLITS), static_cast<const char*>(X), ldx_bytes,
                      static_cast<const char*>(W), ldw_bytes, epi,
-                     static_cast<uint32_t*>(ctx->workspace),
+                     static_cast<uint64_t*>(ctx->workspace),
                      reinterpret_cast<uint32_t*>(static_cast<char*>(ctx->workspace) +
                                                  ctx->ws_partial_bytes));
+}
+
+template <typename Geo, typename Epi>
+void launch_skinny(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
+                   int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
+  const int64_t kts = K / Geo::K_ELEMS;
+  switch (choose_splits<Geo>(ctx, N, kts)) {
+    case 16: launch_skinny_n<Geo, Epi, 16>(ctx, M, N, kts, X, ldx_bytes, W, ldw_bytes, epi); break;
+    case 8: launch_skinny_n<Geo, Epi, 8>(ctx, M, N, kts, X, ldx_bytes, W, ldw_bytes, epi); break;
+    case 4: launch_skinny_n<Geo, Epi, 4>(ctx, M, N, kts, X, ldx_bytes, W, ldw_bytes, epi); break;
+    case 2: launch_skinny_n<Geo, Epi, 2>(ctx, M, N, kts, X, ldx_bytes, W, ldw_bytes, epi); break;
+    default: launch_skinny_n<Geo, Epi, 1>(ctx, M, N, kts, X, ldx_bytes, W, ldw_bytes, epi); break;
+  }
 }
 
 template <typename Geo>
