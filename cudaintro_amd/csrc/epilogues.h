@@ -20,6 +20,15 @@ struct EpiStore16x4 {
   }
 };
 
+struct EpiStoreF32x4 {
+  float* C;
+  int64_t ldc;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float v0, float v1, float v2,
+                                             float v3) const {
+    *reinterpret_cast<f32x4*>(C + r * ldc + c) = f32x4{v0, v1, v2, v3};
+  }
+};
+
 struct EpiStoreI32x4 {
   int32_t* C;
   int64_t ldc;

@@ -1,6 +1,18 @@
-// fp32 GEMM placeholder gate: no MFMA family yet, every shape goes to the any-shape kernel.
-#include "common.h"
+// fp32 GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32: fp32 products, fp32
+// accumulation): the shared LDS-tiled MFMA kernel with the fp32 fragment plumbing.
+#include "epilogues.h"
+#include "mfma_tile.h"
+
 namespace cig {
-bool launch_f32_mfma(cigemmContext*, int64_t, int64_t, int64_t, const float*, int64_t,
-                     const float*, int64_t, float*, int64_t) { return false; }
+
+bool launch_f32_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const float* A,
+                     int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc) {
+  if (!tile::tile_shape_ok(M, N, K, 4, A, lda, B, ldb)) return false;
+  if (ldc % 4 || ((uintptr_t)C & 15)) return false;
+  tile::launch_tile<tile::MathF32, tile::B_KN32>(ctx, M, N, K * 4, A, lda * 4, B, ldb * 4,
+                                                 EpiStoreF32x4{C, ldc});
+  ctx->last_kernel = "f32_mfma_256x256x16_ring4";
+  return true;
+}
+
 }  // namespace cig

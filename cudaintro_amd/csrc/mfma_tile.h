@@ -66,7 +66,16 @@ __device__ __forceinline__ int rowmajor_off(int r, int c) {
   return r * KB + ((c ^ rowmajor_swz(r)) << 4);
 }
 
-enum BMode { B_NK = 0, B_KN16 = 1, B_KN8 = 2 };
+enum BMode { B_NK = 0, B_KN16 = 1, B_KN8 = 2, B_KN32 = 3 };
+
+// Fragment plumbing shared by the 16-bit / int8 tiles: a B fragment is two 8-byte halves.
+struct HalfPieces {
+  static constexpr int NREADS = 8;  // LDS reads per k-step for the four B fragments
+  typedef u32x2 piece_t;
+  static __device__ __forceinline__ u32x4 bfrag(const piece_t (&b)[NREADS], int j, int) {
+    return __builtin_shufflevector(b[2 * j], b[2 * j + 1], 0, 1, 2, 3);
+  }
+};
 
 template <int MODE>
 struct BTile;
@@ -86,7 +95,7 @@ struct RowMajorDma {
 
 // Weights N x K: identical to the A tile.
 template <>
-struct BTile<B_NK> : RowMajorDma {
+struct BTile<B_NK> : RowMajorDma, HalfPieces {
   // half h (0/1) of the fragment of column tile j, k-step kk: 8 bytes of k
   static __device__ __forceinline__ u32x2 frag_half(const char* sb, int wn, int j, int kk, int h,
                                                     int l) {
@@ -97,7 +106,7 @@ struct BTile<B_NK> : RowMajorDma {
 
 // K x N halves: [32 k][32 chunks of 8 halves]; one DMA instruction = 2 k-rows.
 template <>
-struct BTile<B_KN16> {
+struct BTile<B_KN16> : HalfPieces {
   static __device__ __forceinline__ int swz(int k) {
     const int k3 = k & 3;
     return (k3 << 2) | ((((k3 >> 1) ^ k3) & 1) << 1);
@@ -120,7 +129,7 @@ struct BTile<B_KN16> {
 
 // K x N bytes: [64 k][16 chunks of 16 bytes]; one DMA instruction = 4 k-rows.
 template <>
-struct BTile<B_KN8> {
+struct BTile<B_KN8> : HalfPieces {
   static __device__ __forceinline__ int swz(int k) {
     return ((k & 7) << 1) | (((k >> 2) ^ (k >> 4)) & 1);
   }
@@ -140,8 +149,46 @@ struct BTile<B_KN8> {
   }
 };
 
+// K x N fp32: [16 k][256 n] floats, rows of 1 KiB = 64 chunks; one DMA instruction = 1 k-row.
+// Lane (n, g) reads the single float B[k][n] per MFMA; lanes 0-31 and 32-63 read rows k and
+// k+4, which the swizzle moves 128 bytes apart.
+template <>
+struct BTile<B_KN32> {
+  static constexpr int NREADS = 16;
+  typedef uint32_t piece_t;
+  static __device__ __forceinline__ int swz(int k) { return ((k >> 2) & 1) << 3; }
+  static __device__ __forceinline__ int dma_lds(int w, int i) { return (4 * w + i) * 1024; }
+  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
+    const int k = 4 * w + i;
+    return (int64_t)k * ld + ((l ^ swz(k)) << 4);
+  }
+  // read idx (0..15) of k-step kk: element e = idx/4 of the fragment of column tile j = idx%4
+  static __device__ __forceinline__ piece_t read(const char* sb, int wn, int idx, int kk, int l) {
+    const int e = idx >> 2, j = idx & 3;
+    const int k = 8 * kk + 4 * (l >> 5) + e;
+    const int n = wn * 128 + 32 * j + (l & 31);
+    return *reinterpret_cast<const uint32_t*>(sb + k * 1024 + (((n >> 2) ^ swz(k)) << 4) +
+                                              (n & 3) * 4);
+  }
+  static __device__ __forceinline__ float bfrag(const piece_t (&b)[NREADS], int j, int sub) {
+    return __builtin_bit_cast(float, b[4 * sub + j]);
+  }
+};
+
+// read idx (0..7) of k-step kk for the half-piece tiles: half idx%2 of column tile idx/2
+template <int MODE>
+__device__ __forceinline__ typename BTile<MODE>::piece_t read_b_piece(const char* sb, int wn,
+                                                                      int idx, int kk, int l) {
+  if constexpr (MODE == B_KN32)
+    return BTile<MODE>::read(sb, wn, idx, kk, l);
+  else
+    return BTile<MODE>::frag_half(sb, wn, idx >> 1, kk, idx & 1, l);
+}
+
 // ---- arithmetic traits ----------------------------------------------------------------------
 struct MathBF16 {
+  static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
+  static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
   typedef f32x16 acc_t;
   typedef float scalar_t;
   static constexpr int ELEM_BYTES = 2;
@@ -152,6 +199,8 @@ struct MathBF16 {
   }
 };
 struct MathF16 {
+  static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
+  static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
   typedef f32x16 acc_t;
   typedef float scalar_t;
   static constexpr int ELEM_BYTES = 2;
@@ -161,12 +210,31 @@ struct MathF16 {
   }
 };
 struct MathI8 {
+  static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
+  static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
   typedef i32x16 acc_t;
   typedef int32_t scalar_t;
   static constexpr int ELEM_BYTES = 1;
   static __device__ __forceinline__ acc_t mfma(u32x4 first, u32x4 second, acc_t acc) {
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, first),
                                                  __builtin_bit_cast(i32x4, second), acc, 0, 0, 0);
+  }
+};
+
+// fp32: v_mfma_f32_32x32x2_f32 takes one float per lane and operand (row l%32, k = l/32).
+// A 16-byte fragment read gives a lane 4 consecutive k of its row, lanes 32-63 the next 4,
+// so four MFMAs consume one fragment pair: MFMA e multiplies k0+e (lanes 0-31) and k0+4+e.
+struct MathF32 {
+  static constexpr int SUBSTEPS = 4;
+  static __device__ __forceinline__ float afrag(u32x4 a, int sub) {
+    const uint32_t bits = a[sub];  // (bit_cast applied directly to a vector element misreads it)
+    return __builtin_bit_cast(float, bits);
+  }
+  typedef f32x16 acc_t;
+  typedef float scalar_t;
+  static constexpr int ELEM_BYTES = 4;
+  static __device__ __forceinline__ acc_t mfma(float first, float second, acc_t acc) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(first, second, acc, 0, 0, 0);
   }
 };
 
@@ -261,19 +329,20 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
   const int a_frag_row = wm * 128 + (l & 31);
   const int g = l >> 5;
 
-  // One k-step's operands: 4 A fragments (16 B each) and 4 B fragments as 8 halves.
+  // One k-step's operands: 4 A fragments (16 B each) and the pieces of the 4 B fragments.
+  constexpr int NREAD = 4 + BT::NREADS;          // LDS reads per k-step
+  constexpr int NMFMA = 16 * Math::SUBSTEPS;     // MFMAs per k-step
   struct Frags {
     u32x4 a[4];
-    u32x2 b[8];
+    typename BT::piece_t b[BT::NREADS];
   };
-  // LDS read r (0..11) of k-step kk of the stage in ring slot `slot`: 0..3 = A fragment r,
-  // 4..11 = B half.
+  // LDS read r of k-step kk of the stage in ring slot `slot`: 0..3 = A fragment r, then B.
   auto read_piece = [&](Frags& f, int slot, int kk, int r) {
     const char* sa = lds + slot * STAGE_BYTES;
     if (r < 4)
       f.a[r] = *reinterpret_cast<const u32x4*>(sa + rowmajor_off(a_frag_row + 32 * r, 2 * kk + g));
     else
-      f.b[r - 4] = BT::frag_half(sa + OPERAND_BYTES, wn, (r - 4) >> 1, kk, (r - 4) & 1, l);
+      f.b[r - 4] = read_b_piece<BMODE>(sa + OPERAND_BYTES, wn, r - 4, kk, l);
   };
 
   acc_t acc[4][4];
@@ -284,12 +353,11 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  // MFMA m (0..15) of a k-step, column tile j = m/4 outer: the first four need all A
-  // fragments (reads 0..3) but only the first B fragment (reads 4, 5).
+  // MFMA m of a k-step: sub-step m/16 outermost, then column tile j, then row tile i: the
+  // first four need all A fragments (reads 0..3) but only the first pieces of B.
   auto mfma_piece = [&](const Frags& f, int m) {
-    const int j = m >> 2, i = m & 3;
-    const u32x4 bfrag = __builtin_shufflevector(f.b[2 * j], f.b[2 * j + 1], 0, 1, 2, 3);
-    acc[i][j] = Math::mfma(bfrag, f.a[i], acc[i][j]);
+    const int sub = m >> 4, j = (m >> 2) & 3, i = m & 3;
+    acc[i][j] = Math::mfma(BT::bfrag(f.b, j, sub), Math::afrag(f.a[i], sub), acc[i][j]);
   };
 
   Frags f0, f1;
@@ -309,7 +377,7 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int r = 0; r < 12; ++r) read_piece(f0, 0, 0, r);
+  for (int r = 0; r < NREAD; ++r) read_piece(f0, 0, 0, r);
 
   // Ring slots of the stage being multiplied, of the next one, and of the one the DMA fills
   // (wave-uniform scalars, advanced modulo NSTAGES each iteration).
@@ -317,9 +385,9 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
   for (int s = 0; s < KTS; ++s) {
     // k-step 0
 #pragma unroll
-    for (int sl = 0; sl < 16; ++sl) {
+    for (int sl = 0; sl < NMFMA; ++sl) {
       mfma_piece(f0, sl);
-      if (sl < 12) read_piece(f1, slot, 1, sl);
+      if (sl < NREAD) read_piece(f1, slot, 1, sl);
       __builtin_amdgcn_sched_barrier(0);
     }
     // stage s+1 landed for this wave (stages s+2 .. s+DIST-1 may still be in flight)
@@ -328,10 +396,10 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
     __builtin_amdgcn_sched_barrier(0);
     // k-step 1
 #pragma unroll
-    for (int sl = 0; sl < 16; ++sl) {
+    for (int sl = 0; sl < NMFMA; ++sl) {
       mfma_piece(f1, sl);
-      if (sl < 12) read_piece(f0, next_slot, 0, sl);
-      if (sl & 1) dma_piece(s + DIST, dma_slot, sl >> 1);
+      if (sl < NREAD) read_piece(f0, next_slot, 0, sl);
+      if ((sl & 1) && sl < 2 * DMA_PER_STAGE) dma_piece(s + DIST, dma_slot, sl >> 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     slot = next_slot;

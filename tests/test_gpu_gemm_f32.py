@@ -91,3 +91,33 @@ def test_k_zero_and_empty(handle, torch_gpu):
     assert (out.cpu().numpy() == 0).all()          # empty sum
     handle.gemm_f32(torch.empty((0, 3), dtype=torch.float32, device="cuda"),
                     torch.empty((3, 5), dtype=torch.float32, device="cuda"))
+
+
+def test_mfma_path_onehot_and_bound(handle, torch_gpu, oracle, rng):
+    """The fp32 MFMA tile kernel: one-hot rows/columns select exactly, random inputs stay within
+    the fp32 summation bound of fp64, leading dimensions and guard columns are respected."""
+    torch = torch_gpu
+    M, N, K = 512, 768, 272
+    Bf = rng.normal(size=(K, N)).astype(np.float32)
+    perm = rng.integers(0, K, size=M)
+    A = np.zeros((M, K), np.float32)
+    A[np.arange(M), perm] = 1.0
+    C = run(handle, torch, A, Bf)
+    assert "mfma" in handle.last_kernel, handle.last_kernel
+    np.testing.assert_array_equal(C, Bf[perm])
+    Af = rng.normal(size=(M, K)).astype(np.float32)
+    permn = rng.integers(0, K, size=N)
+    B = np.zeros((K, N), np.float32)
+    B[permn, np.arange(N)] = 1.0
+    np.testing.assert_array_equal(run(handle, torch, Af, B), Af[:, permn])
+    # sub-blocks of larger buffers
+    bigA = torch.from_numpy(rng.normal(size=(M, K + 40)).astype(np.float32)).cuda()
+    bigB = torch.from_numpy(rng.normal(size=(K, N + 12)).astype(np.float32)).cuda()
+    out = torch.full((M, N + 8), -3.0, dtype=torch.float32, device="cuda")
+    a, b, c = bigA[:, 8:8 + K], bigB[:, 4:4 + N], out[:, 4:4 + N]
+    handle.gemm_f32(a, b, out=c)
+    assert "mfma" in handle.last_kernel
+    ref, S = oracle.gemm_f64(a.cpu().numpy(), b.cpu().numpy(), with_abs=True)
+    assert (np.abs(c.cpu().numpy() - ref) <= K * 2.0 ** -24 * S).all()
+    o = out.cpu().numpy()
+    assert (o[:, :4] == -3.0).all() and (o[:, 4 + N:] == -3.0).all()
