@@ -1,6 +1,13 @@
-// Epilogue functors shared by the MFMA kernel families.  Each call stores four consecutive
-// columns col..col+3 of one output row.
+// Epilogue functors shared by the MFMA kernel families.  An epilogue turns four consecutive
+// accumulators of one output row (columns col..col+3) into output bits:
+//   pack(row, col, v0..v3)   the 4 output elements as raw bits (u32x2 for 16-bit outputs,
+//                            u32x4 for 32-bit ones), plus any side store (accumulator dump);
+//   out_row(row)             byte address of column 0 of that output row;
+//   operator()               pack + direct store (used where rows are not staged in LDS);
+//   shift_cols(c)            the same epilogue for the sub-problem starting at column c.
 #pragma once
+
+#include <type_traits>
 
 #include "common.h"
 
@@ -11,32 +18,59 @@ template <typename E16>
 struct EpiStore16x4 {
   uint16_t* C;
   int64_t ldc;
-  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float v0, float v1, float v2,
-                                             float v3) const {
+  static constexpr int OUT_BYTES = 2;
+  __device__ __forceinline__ u32x2 pack(int64_t, int64_t, float v0, float v1, float v2,
+                                        float v3) const {
     u32x2 v;
     v[0] = (uint32_t)E16::narrow(v0) | ((uint32_t)E16::narrow(v1) << 16);
     v[1] = (uint32_t)E16::narrow(v2) | ((uint32_t)E16::narrow(v3) << 16);
-    *reinterpret_cast<u32x2*>(C + r * ldc + c) = v;
+    return v;
   }
+  __device__ __forceinline__ char* out_row(int64_t r) const {
+    return reinterpret_cast<char*>(C + r * ldc);
+  }
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float v0, float v1, float v2,
+                                             float v3) const {
+    *reinterpret_cast<u32x2*>(C + r * ldc + c) = pack(r, c, v0, v1, v2, v3);
+  }
+  EpiStore16x4 shift_cols(int64_t c0) const { return EpiStore16x4{C + c0, ldc}; }
 };
 
 struct EpiStoreF32x4 {
   float* C;
   int64_t ldc;
+  static constexpr int OUT_BYTES = 4;
+  __device__ __forceinline__ u32x4 pack(int64_t, int64_t, float v0, float v1, float v2,
+                                        float v3) const {
+    return __builtin_bit_cast(u32x4, f32x4{v0, v1, v2, v3});
+  }
+  __device__ __forceinline__ char* out_row(int64_t r) const {
+    return reinterpret_cast<char*>(C + r * ldc);
+  }
   __device__ __forceinline__ void operator()(int64_t r, int64_t c, float v0, float v1, float v2,
                                              float v3) const {
     *reinterpret_cast<f32x4*>(C + r * ldc + c) = f32x4{v0, v1, v2, v3};
   }
+  EpiStoreF32x4 shift_cols(int64_t c0) const { return EpiStoreF32x4{C + c0, ldc}; }
 };
 
 struct EpiStoreI32x4 {
   int32_t* C;
   int64_t ldc;
+  static constexpr int OUT_BYTES = 4;
+  __device__ __forceinline__ u32x4 pack(int64_t, int64_t, int32_t v0, int32_t v1, int32_t v2,
+                                        int32_t v3) const {
+    return __builtin_bit_cast(u32x4, i32x4{v0, v1, v2, v3});
+  }
+  __device__ __forceinline__ char* out_row(int64_t r) const {
+    return reinterpret_cast<char*>(C + r * ldc);
+  }
   __device__ __forceinline__ void operator()(int64_t r, int64_t c, int32_t v0, int32_t v1,
                                              int32_t v2, int32_t v3) const {
     i32x4 v = {v0, v1, v2, v3};
     *reinterpret_cast<i32x4*>(C + r * ldc + c) = v;
   }
+  EpiStoreI32x4 shift_cols(int64_t c0) const { return EpiStoreI32x4{C + c0, ldc}; }
 };
 
 // out = ((float)acc * sA[row]) * sB[col]: two separately rounded fp32 multiplies, then an
@@ -50,8 +84,10 @@ struct EpiDequantX4 {
   int sa_vec, sb_vec;
   int32_t* acc_out;
   int64_t ldacc;
-  __device__ __forceinline__ void operator()(int64_t r, int64_t c, int32_t v0, int32_t v1,
-                                             int32_t v2, int32_t v3) const {
+  static constexpr int OUT_BYTES = OUT_BF16 ? 2 : 4;
+  typedef typename std::conditional<OUT_BF16, u32x2, u32x4>::type packed_t;
+  __device__ __forceinline__ packed_t pack(int64_t r, int64_t c, int32_t v0, int32_t v1,
+                                           int32_t v2, int32_t v3) const {
     const float a = sa[sa_vec ? r : 0];
     f32x4 b;
     if (sb_vec)
@@ -63,19 +99,33 @@ struct EpiDequantX4 {
     o[1] = __fmul_rn(__fmul_rn((float)v1, a), b[1]);
     o[2] = __fmul_rn(__fmul_rn((float)v2, a), b[2]);
     o[3] = __fmul_rn(__fmul_rn((float)v3, a), b[3]);
-    if (OUT_BF16) {
-      u32x2 p;
-      p[0] = (uint32_t)f32_to_bf16_bits(o[0]) | ((uint32_t)f32_to_bf16_bits(o[1]) << 16);
-      p[1] = (uint32_t)f32_to_bf16_bits(o[2]) | ((uint32_t)f32_to_bf16_bits(o[3]) << 16);
-      *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + r * ldo + c) = p;
-    } else {
-      *reinterpret_cast<f32x4*>(static_cast<float*>(out) + r * ldo + c) =
-          f32x4{o[0], o[1], o[2], o[3]};
-    }
     if (DUMP_ACC) {
       i32x4 v = {v0, v1, v2, v3};
       *reinterpret_cast<i32x4*>(acc_out + r * ldacc + c) = v;
     }
+    if constexpr (OUT_BF16) {
+      u32x2 p;
+      p[0] = (uint32_t)f32_to_bf16_bits(o[0]) | ((uint32_t)f32_to_bf16_bits(o[1]) << 16);
+      p[1] = (uint32_t)f32_to_bf16_bits(o[2]) | ((uint32_t)f32_to_bf16_bits(o[3]) << 16);
+      return p;
+    } else {
+      return __builtin_bit_cast(u32x4, f32x4{o[0], o[1], o[2], o[3]});
+    }
+  }
+  __device__ __forceinline__ char* out_row(int64_t r) const {
+    return static_cast<char*>(out) + r * ldo * OUT_BYTES;
+  }
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, int32_t v0, int32_t v1,
+                                             int32_t v2, int32_t v3) const {
+    *reinterpret_cast<packed_t*>(out_row(r) + c * OUT_BYTES) = pack(r, c, v0, v1, v2, v3);
+  }
+  EpiDequantX4 shift_cols(int64_t c0) const {
+    EpiDequantX4 e = *this;
+    e.out = OUT_BF16 ? static_cast<void*>(static_cast<uint16_t*>(out) + c0)
+                     : static_cast<void*>(static_cast<float*>(out) + c0);
+    if (sb_vec) e.sb = sb + c0;
+    if (DUMP_ACC) e.acc_out = acc_out + c0;
+    return e;
   }
 };
 

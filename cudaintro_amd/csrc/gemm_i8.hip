@@ -38,9 +38,8 @@ bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const i
   if (!dq) {
     if (ldc % 4 || ((uintptr_t)C & 15)) return false;
   } else {
-    if (dq->out_bf16 ? (dq->ldo % 4 || ((uintptr_t)dq->out & 7))
-                     : (dq->ldo % 4 || ((uintptr_t)dq->out & 15)))
-      return false;
+    if (dq->ldo % (dq->out_bf16 ? 8 : 4) || ((uintptr_t)dq->out & 15))
+      return false;  // output rows are stored in 16-byte pieces
     if (dq->sb_vec && ((uintptr_t)dq->sb & 15)) return false;
     if (dq->acc_out && (dq->ldacc % 4 || ((uintptr_t)dq->acc_out & 15))) return false;
   }

@@ -1,9 +1,11 @@
 // The LDS-tiled MFMA GEMM kernel shared by the bf16, fp16 and int8 families.
 //
 // Workgroup = 256 lanes = 4 waves (2 x 2); macro tile 256 (m) x 256 (n); k is consumed in
-// stages of 64 BYTES per row (32 halves or 64 int8) = two MFMA k-steps.  Each wave owns a
-// 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulators per lane (the AGPR file);
-// one wave per SIMD.  Both operand tiles of a stage are 16 KiB; NSTAGES (4 or 5) stages form
+// stages of 64 BYTES per row (32 halves, 64 int8 or 16 floats) = two MFMA k-steps.  Each wave
+// owns a 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulators per lane (the AGPR
+// file); one wave per SIMD.  The tile height is a template parameter (MT = 4, 2 or 1 row
+// tiles per wave: 256, 128 or 64 rows) so that small or awkward M still fill the chip; the
+// text below describes MT = 4.  Both operand tiles of a stage are 16 KiB; NSTAGES (4 or 5) stages form
 // a ring in LDS (128 or 160 KiB), NSTAGES-1 of them in flight ahead of the one being
 // multiplied: HBM/L2 latency here is of the order of a microsecond, two to three stage times.
 //
@@ -51,7 +53,6 @@ constexpr int BM = 256, BN = 256;
 constexpr int KB = 64;                     // bytes of k per stage, per row
 constexpr int OPERAND_BYTES = 256 * KB;    // 16 KiB, either operand
 constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
-constexpr int DMA_PER_STAGE = 8;           // per wave: 4 A + 4 B instructions of 1 KiB
 
 typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
@@ -84,14 +85,16 @@ struct BTile;
 // LDS starting at dma_lds(w, i); lane l fetches the 16 bytes at global byte offset
 // dma_src(w, i, l, ld) from the tile's origin (row stride ld bytes).
 
-// [256 rows][64 B]: one instruction = 16 rows.
-struct RowMajorDma {
-  static __device__ __forceinline__ int dma_lds(int w, int i) { return (64 * w + 16 * i) * KB; }
+// [64 T rows][64 B]: one instruction = 16 rows, wave w moves rows 16 T w .. 16 T (w + 1).
+template <int T>
+struct RowMajorDmaT {
+  static __device__ __forceinline__ int dma_lds(int w, int i) { return (16 * T * w + 16 * i) * KB; }
   static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
-    const int r = 64 * w + 16 * i + (l >> 2);
+    const int r = 16 * T * w + 16 * i + (l >> 2);
     return (int64_t)r * ld + (((l & 3) ^ rowmajor_swz(r)) << 4);
   }
 };
+typedef RowMajorDmaT<4> RowMajorDma;
 
 // Weights N x K: identical to the A tile.
 template <>
@@ -267,7 +270,7 @@ __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int&
 // A, B are byte pointers; lda/ldb are in BYTES.  K_bytes = K * ELEM_BYTES is a multiple of
 // 64, M and N multiples of 256, all rows 16-byte aligned (the launcher checks).  KTS = number
 // of 64-byte stages.
-template <typename Math, int BMODE, int NSTAGES, typename Epi>
+template <typename Math, int BMODE, int NSTAGES, int MT, typename Epi>
 __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tiles_n, int KTS,
                                                            const char* __restrict__ A,
                                                            int64_t lda,
@@ -276,6 +279,9 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
   typedef typename Math::acc_t acc_t;
   typedef BTile<BMODE> BT;
   constexpr int DIST = NSTAGES - 1;  // stages in flight ahead of the one being multiplied
+  constexpr int TILE_M = 64 * MT;    // rows of the macro tile
+  constexpr int DMA_PER_STAGE = MT + 4;  // per wave: MT A + 4 B instructions of 1 KiB
+  typedef RowMajorDmaT<MT> ADma;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int t = threadIdx.x;
   const int l = t & 63;
@@ -284,7 +290,7 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
 
   int tm, tn;
   tile_of_workgroup(tiles_m, tiles_n, tm, tn);
-  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+  const int64_t m0 = (int64_t)tm * TILE_M, n0 = (int64_t)tn * BN;
 
   // ---- DMA sources: uniform tile origin + per-lane byte offsets ------------------------------
   const char* a_tile = A + m0 * lda;  // + stage * KB
@@ -297,12 +303,11 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
     b_tile = B + n0 * Math::ELEM_BYTES;
     b_kstep = (int64_t)(KB / Math::ELEM_BYTES) * ldb;
   }
-  uint32_t a_voff[4], b_voff[4];
+  uint32_t a_voff[MT], b_voff[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    a_voff[i] = (uint32_t)RowMajorDma::dma_src(w, i, l, lda);
-    b_voff[i] = (uint32_t)BT::dma_src(w, i, l, ldb);
-  }
+  for (int i = 0; i < MT; ++i) a_voff[i] = (uint32_t)ADma::dma_src(w, i, l, lda);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) b_voff[i] = (uint32_t)BT::dma_src(w, i, l, ldb);
 
   // The DMA instructions are written as asm so that the compiler's wait-count insertion does
   // not know them: it would otherwise make every later LDS read it cannot tell apart (the
@@ -316,50 +321,51 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
                  : "s"(lds_dst), "v"(src)
                  : "m0");
   };
-  // DMA instruction d (0..7) of stage `st` into ring slot `slot`: even d = A, odd d = B.
+  // DMA instruction d of stage `st` into ring slot `slot`: first the 4 of B, then the MT of A.
   // Past the last stage the last one is fetched again (into a slot nobody reads any more),
   // which keeps the number of outstanding instructions, and so the vmcnt waits, uniform.
   auto dma_piece = [&](int st, int slot, int d) {
     st = st < KTS ? st : KTS - 1;
     const uint32_t sa = lds_base + slot * STAGE_BYTES;
-    const int i = d >> 1;
-    if (d & 1)
-      dma16(b_tile + (int64_t)st * b_kstep + b_voff[i], sa + OPERAND_BYTES + BT::dma_lds(w, i));
+    if (d < 4)
+      dma16(b_tile + (int64_t)st * b_kstep + b_voff[d], sa + OPERAND_BYTES + BT::dma_lds(w, d));
     else
-      dma16(a_tile + (int64_t)st * KB + a_voff[i], sa + RowMajorDma::dma_lds(w, i));
+      dma16(a_tile + (int64_t)st * KB + a_voff[d - 4], sa + ADma::dma_lds(w, d - 4));
   };
 
-  const int a_frag_row = wm * 128 + (l & 31);
+  const int a_frag_row = wm * 32 * MT + (l & 31);
   const int g = l >> 5;
 
-  // One k-step's operands: 4 A fragments (16 B each) and the pieces of the 4 B fragments.
-  constexpr int NREAD = 4 + BT::NREADS;          // LDS reads per k-step
-  constexpr int NMFMA = 16 * Math::SUBSTEPS;     // MFMAs per k-step
+  // One k-step's operands: MT A fragments (16 B each) and the pieces of the 4 B fragments.
+  constexpr int NREAD = MT + BT::NREADS;               // LDS reads per k-step
+  constexpr int NMFMA = 4 * MT * Math::SUBSTEPS;       // MFMAs per k-step
+  constexpr int READS_PER_SLOT = (NREAD + NMFMA - 1) / NMFMA;
+  constexpr int DMA_PER_SLOT = (DMA_PER_STAGE + NMFMA - 1) / NMFMA;
   struct Frags {
-    u32x4 a[4];
+    u32x4 a[MT];
     typename BT::piece_t b[BT::NREADS];
   };
-  // LDS read r of k-step kk of the stage in ring slot `slot`: 0..3 = A fragment r, then B.
+  // LDS read r of k-step kk of the stage in ring slot `slot`: first the A fragments, then B.
   auto read_piece = [&](Frags& f, int slot, int kk, int r) {
     const char* sa = lds + slot * STAGE_BYTES;
-    if (r < 4)
+    if (r < MT)
       f.a[r] = *reinterpret_cast<const u32x4*>(sa + rowmajor_off(a_frag_row + 32 * r, 2 * kk + g));
     else
-      f.b[r - 4] = read_b_piece<BMODE>(sa + OPERAND_BYTES, wn, r - 4, kk, l);
+      f.b[r - MT] = read_b_piece<BMODE>(sa + OPERAND_BYTES, wn, r - MT, kk, l);
   };
 
-  acc_t acc[4][4];
+  acc_t acc[MT][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  // MFMA m of a k-step: sub-step m/16 outermost, then column tile j, then row tile i: the
-  // first four need all A fragments (reads 0..3) but only the first pieces of B.
+  // MFMA m of a k-step: sub-step outermost, then column tile j, then row tile i: the first
+  // MT need all A fragments (the first reads) but only the first pieces of B.
   auto mfma_piece = [&](const Frags& f, int m) {
-    const int sub = m >> 4, j = (m >> 2) & 3, i = m & 3;
+    const int sub = m / (4 * MT), j = (m % (4 * MT)) / MT, i = m % MT;
     acc[i][j] = Math::mfma(BT::bfrag(f.b, j, sub), Math::afrag(f.a[i], sub), acc[i][j]);
   };
 
@@ -390,7 +396,9 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
 #pragma unroll
     for (int sl = 0; sl < NMFMA; ++sl) {
       mfma_piece(f0, sl);
-      if (sl < NREAD) read_piece(f1, slot, 1, sl);
+#pragma unroll
+      for (int r = sl * READS_PER_SLOT; r < (sl + 1) * READS_PER_SLOT; ++r)
+        if (r < NREAD) read_piece(f1, slot, 1, r);
       __builtin_amdgcn_sched_barrier(0);
     }
     // stage s+1 landed for this wave (stages s+2 .. s+DIST-1 may still be in flight)
@@ -401,8 +409,12 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
 #pragma unroll
     for (int sl = 0; sl < NMFMA; ++sl) {
       mfma_piece(f1, sl);
-      if (sl < NREAD) read_piece(f0, next_slot, 0, sl);
-      if ((sl & 1) && sl < 2 * DMA_PER_STAGE) dma_piece(s + DIST, dma_slot, sl >> 1);
+#pragma unroll
+      for (int r = sl * READS_PER_SLOT; r < (sl + 1) * READS_PER_SLOT; ++r)
+        if (r < NREAD) read_piece(f0, next_slot, 0, r);
+#pragma unroll
+      for (int d = sl * DMA_PER_SLOT; d < (sl + 1) * DMA_PER_SLOT; ++d)
+        if (d < DMA_PER_STAGE) dma_piece(s + DIST, dma_slot, d);
       __builtin_amdgcn_sched_barrier(0);
     }
     slot = next_slot;
@@ -410,38 +422,127 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
     dma_slot = dma_slot + 1 == NSTAGES ? 0 : dma_slot + 1;
   }
   wait_vmcnt(std::integral_constant<int, 0>{});  // no DMA outlives the main loop
+  __syncthreads();  // ... for any wave, and every wave is done reading the ring
 
-  // acc[i][j][4q+e] = C[m0 + wm*128 + 32i + l%32][n0 + wn*128 + 32j + 8q + 4g + e]
+  // ---- epilogue -----------------------------------------------------------------------------
+  // acc[i][j][4q+e] = C[m0 + wm*32*MT + 32i + l%32][n0 + wn*128 + 32j + 8q + 4g + e]: a lane
+  // holds short pieces of 32 different rows.  Each wave stages one 32-row x 128-column block
+  // at a time in its own piece of the (now idle) LDS and writes it out as whole rows: every
+  // store instruction then covers full 256- or 512-byte row segments.
+  constexpr int OB = Epi::OUT_BYTES;
+  constexpr int ROW_BYTES = 128 * OB;
+  constexpr int ROW_STRIDE = ROW_BYTES + 16;
+  constexpr int LANES_PER_ROW = ROW_BYTES / 16;
+  constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+  char* scr = lds + w * (32 * ROW_STRIDE);
+  typedef decltype(epi.pack(0, 0, acc[0][0][0], acc[0][0][0], acc[0][0][0], acc[0][0][0])) packed_t;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int64_t row = m0 + wm * 128 + 32 * i + (l & 31);
+  for (int i = 0; i < MT; ++i) {
+    const int64_t row0 = m0 + wm * 32 * MT + 32 * i;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        epi(row, n0 + wn * 128 + 32 * j + 8 * q + 4 * g, acc[i][j][4 * q + 0],
-            acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+      for (int q = 0; q < 4; ++q) {
+        const int c = 32 * j + 8 * q + 4 * g;
+        *reinterpret_cast<packed_t*>(scr + (l & 31) * ROW_STRIDE + c * OB) =
+            epi.pack(row0 + (l & 31), n0 + wn * 128 + c, acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
+                     acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+      }
+#pragma unroll
+    for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
+      const int rl = p * ROWS_PER_PASS + l / LANES_PER_ROW;
+      const int c16 = l % LANES_PER_ROW;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(scr + rl * ROW_STRIDE + c16 * 16);
+      *reinterpret_cast<u32x4*>(epi.out_row(row0 + rl) + (n0 + wn * 128) * OB + c16 * 16) = v;
+    }
   }
 }
 
 constexpr int DEFAULT_STAGES = 4;
 
-template <typename Math, int BMODE, typename Epi, int NSTAGES = DEFAULT_STAGES>
-void launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
-                 int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi) {
-  static_assert(NSTAGES == 4 || NSTAGES == 5, "ring of 4 or 5 stages");
+template <typename Math, int BMODE, int MT, typename Epi>
+void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
+                    int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi) {
+  constexpr int NSTAGES = DEFAULT_STAGES;
   constexpr int LDS_BYTES = NSTAGES * STAGE_BYTES;
-  auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, Epi>;
+  auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, MT, Epi>;
   static int attr_device = -1;  // one per template instance
   if (attr_device != ctx->device) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                               LDS_BYTES);
     attr_device = ctx->device;
   }
-  const int tiles_m = (int)(M / BM), tiles_n = (int)(N / BN);
+  const int tiles_m = (int)(M / (64 * MT)), tiles_n = (int)(N / BN);
   hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), LDS_BYTES, ctx->stream,
                      tiles_m, tiles_n, (int)(K_bytes / KB), static_cast<const char*>(A),
                      lda_bytes, static_cast<const char*>(B), ldb_bytes, epi);
+}
+
+// Relative cost of covering M x N with tiles of 64*mt rows on `cus` compute units: rounds of
+// workgroups times the cost of one tile; shorter tiles re-read B more often per flop.
+inline double tile_plan_cost(int64_t M, int64_t N, int mt, int cus) {
+  if (M % (64 * mt)) return 1e30;
+  const int64_t tiles = (M / (64 * mt)) * (N / BN);
+  const double per_tile = mt == 4 ? 4.0 : mt == 2 ? 2.0 * 1.12 : 1.0 * 1.3;
+  return (double)((tiles + cus - 1) / cus) * per_tile;
+}
+inline int best_mt(int64_t M, int64_t N, int cus, double* cost = nullptr) {
+  int best = 0;
+  double bc = 1e30;
+  for (int mt : {4, 2, 1}) {
+    const double c = tile_plan_cost(M, N, mt, cus);
+    if (c < bc) {
+      bc = c;
+      best = mt;
+    }
+  }
+  if (cost) *cost = bc;
+  return best;
+}
+
+template <typename Math, int BMODE, typename Epi>
+void launch_tile_any_mt(cigemmContext* ctx, int mt, int64_t M, int64_t N, int64_t K_bytes,
+                        const void* A, int64_t lda_bytes, const void* B, int64_t ldb_bytes,
+                        const Epi& epi) {
+  if (mt == 4)
+    launch_tile_mt<Math, BMODE, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+  else if (mt == 2)
+    launch_tile_mt<Math, BMODE, 2>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+  else
+    launch_tile_mt<Math, BMODE, 1>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+}
+
+// Chooses the tile height, and, when the last round of 256-row tiles would leave most of the
+// chip idle, covers the columns of the full rounds with 256-row tiles and the remaining
+// columns with a second launch of shorter tiles.  Epi::shift_cols(c) returns the epilogue of
+// the sub-problem starting at column c.
+template <typename Math, int BMODE, typename Epi>
+void launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
+                 int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi) {
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  double single = 0;
+  const int mt = best_mt(M, N, cus, &single);
+  if (M % BM == 0) {
+    const int64_t tiles_m = M / BM, tiles_n = N / BN;
+    if (tiles_m * tiles_n > cus && cus % tiles_m == 0) {
+      const int64_t cols_per_round = cus / tiles_m;
+      const int64_t full_cols = (tiles_n / cols_per_round) * cols_per_round;
+      if (full_cols > 0 && full_cols < tiles_n) {
+        const int64_t n1 = full_cols * BN, n2 = N - n1;
+        double rest = 0;
+        const int mt2 = best_mt(M, n2, cus, &rest);
+        if (tile_plan_cost(M, n1, 4, cus) + rest < single * 0.97) {
+          launch_tile_mt<Math, BMODE, 4>(ctx, M, n1, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+          const char* B2 = static_cast<const char*>(B) +
+                           (BMODE == B_NK ? n1 * ldb_bytes : n1 * Math::ELEM_BYTES);
+          launch_tile_any_mt<Math, BMODE>(ctx, mt2, M, n2, K_bytes, A, lda_bytes, B2, ldb_bytes,
+                                          epi.shift_cols(n1));
+          return;
+        }
+      }
+    }
+  }
+  launch_tile_any_mt<Math, BMODE>(ctx, mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
 }
 
 // Shape / alignment gate shared by the families (sizes in elements, elem = bytes each).
@@ -449,10 +550,10 @@ void launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
 inline bool tile_shape_ok(int64_t M, int64_t N, int64_t K, int elem, const void* A, int64_t lda,
                           const void* B, int64_t ldb) {
   if (M <= 0 || N <= 0 || K <= 0) return false;
-  if (M % BM || N % BN || (K * elem) % KB) return false;
+  if (M % 64 || N % BN || (K * elem) % KB) return false;
   if ((lda * elem) % 16 || (ldb * elem) % 16) return false;
   if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return false;
-  if ((M / BM) * (N / BN) > 2147483647LL) return false;
+  if ((M / 64) * (N / BN) > 2147483647LL) return false;
   if (lda * elem * 256 >= (1LL << 32) || ldb * elem * 256 >= (1LL << 32)) return false;
   return true;
 }

@@ -40,7 +40,8 @@ def check_bound(oracle, Cb, Ab, Bb, kind, rows=None):
 
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(256, 256, 64), (256, 256, 128), (512, 256, 192), (256, 768, 1024),
-                                   (1024, 1024, 1024)])
+                                   (1024, 1024, 1024), (64, 256, 32), (128, 512, 96), (192, 256, 160),
+                                   (320, 1024, 64), (2048, 2816, 128)])
 def test_exact_inputs_bit_exact_mfma(handle, torch_gpu, oracle, rng, kind, shape):
     """Inputs from {0, +-0.5, +-1, +-2}: every partial sum is exact in fp32, so the result
     does not depend on summation order and must equal the CPU loop bit for bit."""
@@ -92,13 +93,18 @@ def test_leading_dimensions(handle, torch_gpu, oracle, rng, kind):
     bigA, bigB = to_dev(torch, Ab, kind), to_dev(torch, Bb, kind)
     a = bigA[:M, 8:8 + K]           # lda = K + 72
     b = bigB[:K, 16:16 + N]         # ldb = N + 24
-    out = torch.zeros((M, N + 8), dtype=bigA.dtype, device="cuda")
-    c = out[:, 4:4 + N]
+    out = torch.zeros((M, N + 16), dtype=bigA.dtype, device="cuda")
+    c = out[:, 8:8 + N]
     (handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16)(a, b, out=c)
     assert "mfma" in handle.last_kernel
     check_bound(oracle, bits(torch, c), bits(torch, a), bits(torch, b), kind)
     o = bits(torch, out)
-    assert (o[:, :4] == 0).all() and (o[:, 4 + N:] == 0).all()
+    assert (o[:, :8] == 0).all() and (o[:, 8 + N:] == 0).all()
+    # an output whose rows are only 8-byte aligned is still served (by the any-shape kernel)
+    out2 = torch.zeros((M, N + 8), dtype=bigA.dtype, device="cuda")
+    c2 = out2[:, 4:4 + N]
+    (handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16)(a, b, out=c2)
+    check_bound(oracle, bits(torch, c2), bits(torch, a), bits(torch, b), kind)
 
 
 @pytest.mark.parametrize("kind", KINDS)

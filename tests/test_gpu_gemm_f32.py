@@ -46,7 +46,8 @@ def test_ragged_shapes(handle, torch_gpu, oracle, rng, M, N, K):
 
 def test_exact_inputs_are_bit_exact(handle, torch_gpu, oracle, rng):
     vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
-    for (M, N, K) in [(64, 64, 64), (256, 256, 256), (130, 70, 1000), (512, 512, 512)]:
+    for (M, N, K) in [(64, 64, 64), (256, 256, 256), (130, 70, 1000), (512, 512, 512), (64, 256, 16),
+                      (192, 512, 48), (2048, 2816, 32)]:
         A = rng.choice(vals, size=(M, K))
         B = rng.choice(vals, size=(K, N))
         np.testing.assert_array_equal(run(handle, torch_gpu, A, B), oracle.gemm_f32(A, B))
