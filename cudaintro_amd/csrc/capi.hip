@@ -161,8 +161,9 @@ static cigemmStatus_t gemm16(cigemmHandle_t h, const char* name, bool bf16, int6
   if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
   cigemmStatus_t st = check_gemm_args(h, name, M, N, K, A, lda, B, ldb, N, C, ldc);
   if (st != CIGEMM_STATUS_SUCCESS || M == 0 || N == 0) return st;
-  if (!launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc) &&
-      !launch_skinny_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc))
+  // decode shapes (M <= 32) first: they are bandwidth problems with their own kernel
+  if (!launch_skinny_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc) &&
+      !launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc))
     launch_generic_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc);
   return check_launch(h, name);
 }
@@ -184,8 +185,8 @@ static cigemmStatus_t gemm_i8(cigemmHandle_t h, const char* name, int64_t M, int
                               cigemmBLayout_t b_layout, int32_t* C, int64_t ldc,
                               const DequantArgs* dq) {
   const bool b_nk = b_layout == CIGEMM_B_NK;
-  if (!launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq) &&
-      !launch_skinny_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq))
+  if (!launch_skinny_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq) &&
+      !launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq))
     launch_generic_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);
   return check_launch(h, name);
 }

@@ -1,7 +1,8 @@
 // Epilogue functors shared by the MFMA kernel families.  An epilogue turns four consecutive
 // accumulators of one output row (columns col..col+3) into output bits:
 //   pack(row, col, v0..v3)   the 4 output elements as raw bits (u32x2 for 16-bit outputs,
-//                            u32x4 for 32-bit ones), plus any side store (accumulator dump);
+//                            u32x4 for 32-bit ones); no memory is written;
+//   side(row, col, v0..v3)   any second output of the same quad (the accumulator dump);
 //   out_row(row)             byte address of column 0 of that output row;
 //   operator()               pack + direct store (used where rows are not staged in LDS);
 //   shift_cols(c)            the same epilogue for the sub-problem starting at column c.
@@ -33,6 +34,7 @@ struct EpiStore16x4 {
                                              float v3) const {
     *reinterpret_cast<u32x2*>(C + r * ldc + c) = pack(r, c, v0, v1, v2, v3);
   }
+  __device__ __forceinline__ void side(int64_t, int64_t, float, float, float, float) const {}
   EpiStore16x4 shift_cols(int64_t c0) const { return EpiStore16x4{C + c0, ldc}; }
 };
 
@@ -51,6 +53,7 @@ struct EpiStoreF32x4 {
                                              float v3) const {
     *reinterpret_cast<f32x4*>(C + r * ldc + c) = f32x4{v0, v1, v2, v3};
   }
+  __device__ __forceinline__ void side(int64_t, int64_t, float, float, float, float) const {}
   EpiStoreF32x4 shift_cols(int64_t c0) const { return EpiStoreF32x4{C + c0, ldc}; }
 };
 
@@ -70,6 +73,7 @@ struct EpiStoreI32x4 {
     i32x4 v = {v0, v1, v2, v3};
     *reinterpret_cast<i32x4*>(C + r * ldc + c) = v;
   }
+  __device__ __forceinline__ void side(int64_t, int64_t, int32_t, int32_t, int32_t, int32_t) const {}
   EpiStoreI32x4 shift_cols(int64_t c0) const { return EpiStoreI32x4{C + c0, ldc}; }
 };
 
@@ -99,10 +103,6 @@ struct EpiDequantX4 {
     o[1] = __fmul_rn(__fmul_rn((float)v1, a), b[1]);
     o[2] = __fmul_rn(__fmul_rn((float)v2, a), b[2]);
     o[3] = __fmul_rn(__fmul_rn((float)v3, a), b[3]);
-    if (DUMP_ACC) {
-      i32x4 v = {v0, v1, v2, v3};
-      *reinterpret_cast<i32x4*>(acc_out + r * ldacc + c) = v;
-    }
     if constexpr (OUT_BF16) {
       u32x2 p;
       p[0] = (uint32_t)f32_to_bf16_bits(o[0]) | ((uint32_t)f32_to_bf16_bits(o[1]) << 16);
@@ -115,9 +115,17 @@ struct EpiDequantX4 {
   __device__ __forceinline__ char* out_row(int64_t r) const {
     return static_cast<char*>(out) + r * ldo * OUT_BYTES;
   }
+  __device__ __forceinline__ void side(int64_t r, int64_t c, int32_t v0, int32_t v1, int32_t v2,
+                                       int32_t v3) const {
+    if (DUMP_ACC) {
+      i32x4 v = {v0, v1, v2, v3};
+      *reinterpret_cast<i32x4*>(acc_out + r * ldacc + c) = v;
+    }
+  }
   __device__ __forceinline__ void operator()(int64_t r, int64_t c, int32_t v0, int32_t v1,
                                              int32_t v2, int32_t v3) const {
     *reinterpret_cast<packed_t*>(out_row(r) + c * OUT_BYTES) = pack(r, c, v0, v1, v2, v3);
+    side(r, c, v0, v1, v2, v3);
   }
   EpiDequantX4 shift_cols(int64_t c0) const {
     EpiDequantX4 e = *this;

@@ -7,7 +7,7 @@ namespace cig {
 
 bool launch_f32_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const float* A,
                      int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc) {
-  if (!tile::tile_shape_ok(M, N, K, 4, A, lda, B, ldb)) return false;
+  if (!tile::tile_shape_ok(M, N, K, 4, A, lda, B, ldb, true)) return false;
   if (ldc % 4 || ((uintptr_t)C & 15)) return false;
   tile::launch_tile<tile::MathF32, tile::B_KN32>(ctx, M, N, K * 4, A, lda * 4, B, ldb * 4,
                                                  EpiStoreF32x4{C, ldc});

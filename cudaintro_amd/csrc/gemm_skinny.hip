@@ -59,7 +59,7 @@ struct GeoKN16 {
                                              int M, uint32_t slot_lds, int w, int l) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      dma16(W + WT::dma_src(w, i, l, ldw), slot_lds + WT::dma_lds(w, i));
+      dma16(W + WT::dma_src(w, i, l, ldw, 31), slot_lds + WT::dma_lds(w, i));
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int r = 8 * w + 4 * i + (l >> 4);

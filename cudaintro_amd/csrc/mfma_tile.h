@@ -89,9 +89,10 @@ struct BTile;
 template <int T>
 struct RowMajorDmaT {
   static __device__ __forceinline__ int dma_lds(int w, int i) { return (16 * T * w + 16 * i) * KB; }
-  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
+  // `last` = last valid row of the tile (rows beyond it re-read it; they are never stored)
+  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld, int last) {
     const int r = 16 * T * w + 16 * i + (l >> 2);
-    return (int64_t)r * ld + (((l & 3) ^ rowmajor_swz(r)) << 4);
+    return (int64_t)(r < last ? r : last) * ld + (((l & 3) ^ rowmajor_swz(r)) << 4);
   }
 };
 typedef RowMajorDmaT<4> RowMajorDma;
@@ -116,9 +117,11 @@ struct BTile<B_KN16> : HalfPieces {
   }
   static __device__ __forceinline__ int off(int k, int c) { return k * 512 + ((c ^ swz(k)) << 4); }
   static __device__ __forceinline__ int dma_lds(int w, int i) { return (8 * w + 2 * i) * 512; }
-  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
+  // `last` = last valid 16-byte chunk of a tile row (columns beyond N re-read it)
+  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld, int last) {
     const int k = 8 * w + 2 * i + (l >> 5);
-    return (int64_t)k * ld + (((l & 31) ^ swz(k)) << 4);
+    const int c = (l & 31) ^ swz(k);
+    return (int64_t)k * ld + ((c < last ? c : last) << 4);
   }
   static __device__ __forceinline__ u32x2 frag_half(const char* sb, int wn, int j, int kk, int h,
                                                     int l) {
@@ -138,9 +141,10 @@ struct BTile<B_KN8> : HalfPieces {
   }
   static __device__ __forceinline__ int off(int k, int c) { return k * 256 + ((c ^ swz(k)) << 4); }
   static __device__ __forceinline__ int dma_lds(int w, int i) { return (16 * w + 4 * i) * 256; }
-  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
+  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld, int last) {
     const int k = 16 * w + 4 * i + (l >> 4);
-    return (int64_t)k * ld + (((l & 15) ^ swz(k)) << 4);
+    const int c = (l & 15) ^ swz(k);
+    return (int64_t)k * ld + ((c < last ? c : last) << 4);
   }
   static __device__ __forceinline__ u32x2 frag_half(const char* sb, int wn, int j, int kk, int h,
                                                     int l) {
@@ -161,9 +165,10 @@ struct BTile<B_KN32> {
   typedef uint32_t piece_t;
   static __device__ __forceinline__ int swz(int k) { return ((k >> 2) & 1) << 3; }
   static __device__ __forceinline__ int dma_lds(int w, int i) { return (4 * w + i) * 1024; }
-  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld) {
+  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld, int last) {
     const int k = 4 * w + i;
-    return (int64_t)k * ld + ((l ^ swz(k)) << 4);
+    const int c = l ^ swz(k);
+    return (int64_t)k * ld + ((c < last ? c : last) << 4);
   }
   // read idx (0..15) of k-step kk: element e = idx/4 of the fragment of column tile j = idx%4
   static __device__ __forceinline__ piece_t read(const char* sb, int wn, int idx, int kk, int l) {
@@ -271,7 +276,8 @@ __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int&
 // 64, M and N multiples of 256, all rows 16-byte aligned (the launcher checks).  KTS = number
 // of 64-byte stages.
 template <typename Math, int BMODE, int NSTAGES, int MT, typename Epi>
-__global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tiles_n, int KTS,
+__global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int tiles_m,
+                                                           int tiles_n, int KTS,
                                                            const char* __restrict__ A,
                                                            int64_t lda,
                                                            const char* __restrict__ B,
@@ -303,11 +309,17 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
     b_tile = B + n0 * Math::ELEM_BYTES;
     b_kstep = (int64_t)(KB / Math::ELEM_BYTES) * ldb;
   }
+  // Ragged edges: rows past M (and, for N x K weights, past N) re-read the last valid row,
+  // column chunks past N (K x N operands) re-read the last valid chunk; what they produce
+  // is never stored.
+  const int a_last = (int)((M - 1 - m0) < (TILE_M - 1) ? (M - 1 - m0) : (TILE_M - 1));
+  const int n_left = (int)((N - n0) < BN ? (N - n0) : BN);
+  const int b_last = BMODE == B_NK ? n_left - 1 : n_left * Math::ELEM_BYTES / 16 - 1;
   uint32_t a_voff[MT], b_voff[4];
 #pragma unroll
-  for (int i = 0; i < MT; ++i) a_voff[i] = (uint32_t)ADma::dma_src(w, i, l, lda);
+  for (int i = 0; i < MT; ++i) a_voff[i] = (uint32_t)ADma::dma_src(w, i, l, lda, a_last);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) b_voff[i] = (uint32_t)BT::dma_src(w, i, l, ldb);
+  for (int i = 0; i < 4; ++i) b_voff[i] = (uint32_t)BT::dma_src(w, i, l, ldb, b_last);
 
   // The DMA instructions are written as asm so that the compiler's wait-count insertion does
   // not know them: it would otherwise make every later LDS read it cannot tell apart (the
@@ -439,21 +451,31 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int tiles_m, int tile
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     const int64_t row0 = m0 + wm * 32 * MT + 32 * i;
+    const int64_t row = row0 + (l & 31);
+    const bool row_ok = row < M;
+    const int64_t row_c = row_ok ? row : M - 1;  // scale lookups stay in bounds
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int c = 32 * j + 8 * q + 4 * g;
+        const int64_t col = n0 + wn * 128 + c;
+        const bool col_ok = col < N;  // N is a multiple of 4: a quad is in or out as a whole
         *reinterpret_cast<packed_t*>(scr + (l & 31) * ROW_STRIDE + c * OB) =
-            epi.pack(row0 + (l & 31), n0 + wn * 128 + c, acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
+            epi.pack(row_c, col_ok ? col : N - 4, acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
                      acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        if (row_ok && col_ok)
+          epi.side(row, col, acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                   acc[i][j][4 * q + 3]);
       }
 #pragma unroll
     for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
       const int rl = p * ROWS_PER_PASS + l / LANES_PER_ROW;
       const int c16 = l % LANES_PER_ROW;
       const u32x4 v = *reinterpret_cast<const u32x4*>(scr + rl * ROW_STRIDE + c16 * 16);
-      *reinterpret_cast<u32x4*>(epi.out_row(row0 + rl) + (n0 + wn * 128) * OB + c16 * 16) = v;
+      // N * OB is a multiple of 16: a 16-byte piece is in or out as a whole
+      if (row0 + rl < M && n0 + wn * 128 + c16 * (16 / OB) < N)
+        *reinterpret_cast<u32x4*>(epi.out_row(row0 + rl) + (n0 + wn * 128) * OB + c16 * 16) = v;
     }
   }
 }
@@ -472,17 +494,17 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
                               LDS_BYTES);
     attr_device = ctx->device;
   }
-  const int tiles_m = (int)(M / (64 * MT)), tiles_n = (int)(N / BN);
+  const int tiles_m = (int)((M + 64 * MT - 1) / (64 * MT)), tiles_n = (int)((N + BN - 1) / BN);
   hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), LDS_BYTES, ctx->stream,
-                     tiles_m, tiles_n, (int)(K_bytes / KB), static_cast<const char*>(A),
+                     (int)M, (int)N, tiles_m, tiles_n, (int)(K_bytes / KB),
+                     static_cast<const char*>(A),
                      lda_bytes, static_cast<const char*>(B), ldb_bytes, epi);
 }
 
 // Relative cost of covering M x N with tiles of 64*mt rows on `cus` compute units: rounds of
 // workgroups times the cost of one tile; shorter tiles re-read B more often per flop.
 inline double tile_plan_cost(int64_t M, int64_t N, int mt, int cus) {
-  if (M % (64 * mt)) return 1e30;
-  const int64_t tiles = (M / (64 * mt)) * (N / BN);
+  const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + BN - 1) / BN);
   const double per_tile = mt == 4 ? 4.0 : mt == 2 ? 2.0 * 1.12 : 1.0 * 1.3;
   return (double)((tiles + cus - 1) / cus) * per_tile;
 }
@@ -522,8 +544,8 @@ void launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
   double single = 0;
   const int mt = best_mt(M, N, cus, &single);
-  if (M % BM == 0) {
-    const int64_t tiles_m = M / BM, tiles_n = N / BN;
+  {
+    const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > cus && cus % tiles_m == 0) {
       const int64_t cols_per_round = cus / tiles_m;
       const int64_t full_cols = (tiles_n / cols_per_round) * cols_per_round;
@@ -545,15 +567,20 @@ void launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
   launch_tile_any_mt<Math, BMODE>(ctx, mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
 }
 
-// Shape / alignment gate shared by the families (sizes in elements, elem = bytes each).
-// Per-lane DMA offsets are 32-bit: 256 rows of either operand must span less than 4 GiB.
+// Shape / alignment gate shared by the families (sizes in elements, elem = bytes each;
+// b_kn = B is K x N).  M is free; K must fill whole 64-byte stages (nothing pads k with
+// zeros); N must keep 16-byte pieces whole, on the input side (K x N rows) and on the output
+// side (the caller checks its output type).  Per-lane DMA offsets are 32-bit: 256 rows of
+// either operand must span less than 4 GiB.
 inline bool tile_shape_ok(int64_t M, int64_t N, int64_t K, int elem, const void* A, int64_t lda,
-                          const void* B, int64_t ldb) {
+                          const void* B, int64_t ldb, bool b_kn) {
   if (M <= 0 || N <= 0 || K <= 0) return false;
-  if (M % 64 || N % BN || (K * elem) % KB) return false;
+  if ((K * elem) % KB || N % 4) return false;
+  if (b_kn && (N * elem) % 16) return false;
+  if (M > 2147483647LL || N > 2147483647LL) return false;
   if ((lda * elem) % 16 || (ldb * elem) % 16) return false;
   if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return false;
-  if ((M / 64) * (N / BN) > 2147483647LL) return false;
+  if (((M + 63) / 64) * ((N + BN - 1) / BN) > 2147483647LL) return false;
   if (lda * elem * 256 >= (1LL << 32) || ldb * elem * 256 >= (1LL << 32)) return false;
   return true;
 }

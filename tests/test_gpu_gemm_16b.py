@@ -77,11 +77,14 @@ def test_onehot_selects_rows_and_columns(handle, torch_gpu, oracle, rng, kind):
 
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("shape", [(256, 256, 512), (512, 768, 2048), (1, 1, 1), (3, 7, 17), (33, 65, 129),
-                                   (129, 17, 65), (255, 257, 63), (64, 64, 4096)])
+                                   (129, 17, 65), (255, 257, 63), (64, 64, 4096), (33, 8, 32), (100, 264, 96),
+                                   (257, 1032, 160), (5000, 520, 64), (333, 40, 2048)])
 def test_random_within_bound(handle, torch_gpu, oracle, kind, shape):
     M, N, K = shape
     Ab, Bb = wl.normal_16bit(M, N, K, seed=7, kind=kind)
     Cb = run(handle, torch_gpu, Ab, Bb, kind)
+    if M > 32 and N % 8 == 0 and K % 32 == 0:
+        assert "mfma" in handle.last_kernel, handle.last_kernel
     check_bound(oracle, Cb, Ab, Bb, kind)
 
 

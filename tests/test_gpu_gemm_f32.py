@@ -122,3 +122,20 @@ def test_mfma_path_onehot_and_bound(handle, torch_gpu, oracle, rng):
     assert (np.abs(c.cpu().numpy() - ref) <= K * 2.0 ** -24 * S).all()
     o = out.cpu().numpy()
     assert (o[:, :4] == -3.0).all() and (o[:, 4 + N:] == -3.0).all()
+
+
+@pytest.mark.parametrize("shape", [(33, 4, 16), (100, 260, 48), (257, 1028, 64), (20000, 512, 784), (1000, 12, 512)])
+def test_mfma_path_ragged_shapes(handle, torch_gpu, oracle, rng, shape):
+    """Any M, N a multiple of 4, K a multiple of 16 go through the MFMA tile kernel with
+    clamped loads and masked stores; guard rows/columns of the output stay untouched."""
+    torch = torch_gpu
+    M, N, K = shape
+    A = rng.uniform(-1, 1, size=(M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, size=(K, N)).astype(np.float32)
+    out = torch.full((M + 3, N + 4), -9.0, dtype=torch.float32, device="cuda")
+    handle.gemm_f32(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), out=out[:M, :N])
+    assert "mfma" in handle.last_kernel, handle.last_kernel
+    o = out.cpu().numpy()
+    ref, S = oracle.gemm_f64(A, B, with_abs=True)
+    assert (np.abs(o[:M, :N] - ref) <= K * 2.0 ** -24 * S + 1e-30).all()
+    assert (o[M:] == -9.0).all() and (o[:, N:] == -9.0).all()

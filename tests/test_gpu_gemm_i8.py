@@ -18,15 +18,16 @@ def dev(torch, a):
 @pytest.mark.parametrize("shape", [(1, 1, 1), (2, 3, 7), (17, 33, 65), (129, 65, 33), (64, 64, 4096),
                                    (255, 257, 127), (256, 256, 128), (256, 512, 384), (768, 256, 1024),
                                    (1024, 1024, 1024), (64, 256, 64), (128, 512, 192), (192, 256, 320),
-                                   (320, 768, 128), (2048, 2816, 256)])
+                                   (320, 768, 128), (2048, 2816, 256), (33, 16, 64), (100, 272, 128), (257, 1040, 192),
+                                   (20000, 512, 64), (500, 48, 4096)])
 def test_accumulators_bit_exact(handle, torch_gpu, oracle, rng, b_nk, shape):
     M, N, K = shape
     A = rng.integers(-128, 128, size=(M, K), dtype=np.int8)
     B = rng.integers(-128, 128, size=(N, K) if b_nk else (K, N), dtype=np.int8)
     C = handle.gemm_i8_i32(dev(torch_gpu, A), dev(torch_gpu, B), ci.B_NK if b_nk else ci.B_KN)
     np.testing.assert_array_equal(C.cpu().numpy(), oracle.gemm_i8_i32(A, B, b_nk))
-    if M % 64 == 0 and N % 256 == 0 and K % 64 == 0:
-        assert "mfma" in handle.last_kernel
+    if M > 32 and N % 16 == 0 and K % 64 == 0:
+        assert "mfma" in handle.last_kernel, handle.last_kernel
 
 
 @pytest.mark.parametrize("b_nk", [False, True])
