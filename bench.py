@@ -213,6 +213,21 @@ def main():
                                         "peak": PEAK_FP32_MATRIX_TFLOPS, "ms": e / steps * 1e3,
                                         "kernel": handle.last_kernel}
 
+        # MLP forward layers of the reference's MNIST demo on the fp32 GEMM with the fused
+        # bias + ReLU epilogue (MNIST/mnist_nn.h:12-15: batch 20000, 784 -> 512 -> 10)
+        r = np.random.Generator(np.random.PCG64(5))
+        for name, (Mb, Kb, Nb), act in (("mnist_hidden_20000x784x512_bias_relu", (20000, 784, 512), ci.ACT_RELU),
+                                        ("mnist_output_20000x512x10_bias", (20000, 512, 10), ci.ACT_NONE)):
+            x = torch.from_numpy(r.uniform(0, 1, size=(Mb, Kb)).astype(np.float32)).cuda()
+            wgt = torch.from_numpy((r.standard_normal((Kb, Nb)) * 0.05).astype(np.float32)).cuda()
+            bias = torch.from_numpy(r.standard_normal(Nb).astype(np.float32)).cuda()
+            o = torch.empty((Mb, Nb), dtype=torch.float32, device="cuda")
+            w_, e = time_calls(torch, lambda: handle.linear_f32(x, wgt, bias, act, out=o), args.steps, 2)
+            t = wl.gemm_ops(Mb, Nb, Kb) * args.steps / e / 1e12
+            per_config[name] = {"tflops": t, "frac_of_peak": t / PEAK_FP32_MATRIX_TFLOPS,
+                                "peak": PEAK_FP32_MATRIX_TFLOPS, "ms": e / args.steps * 1e3,
+                                "kernel": handle.last_kernel}
+
         # skinny decode shapes: HBM-bound.  Rotate over several distinct weight buffers so the
         # working set (> 256 MB) cannot sit in the Infinity Cache between calls.
         for M in (1, 8, 32):

@@ -7,6 +7,8 @@ There is no CPU fallback: importing works anywhere, but creating a handle needs 
 library and a gfx950 device.
 """
 from .cigemm import (  # noqa: F401
+    ACT_NONE,
+    ACT_RELU,
     B_KN,
     B_NK,
     OUT_BF16,

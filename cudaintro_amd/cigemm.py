@@ -16,6 +16,7 @@ _LIB = os.path.join(_HERE, "libcigemm.so")
 _SUITE = os.path.join(_HERE, "gemm_suite")
 
 B_KN, B_NK = 0, 1
+ACT_NONE, ACT_RELU = 0, 1
 SCALE_TENSOR, SCALE_VECTOR = 0, 1
 OUT_F32, OUT_BF16 = 0, 1
 
@@ -72,6 +73,7 @@ SIGNATURES = {
     "cigemm_gemm_i8_i32": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _ci, _vp, _i64]),
     "cigemm_gemm_i8_dequant": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _ci, _vp, _ci,
                                      _vp, _ci, _vp, _ci, _i64, _vp, _i64]),
+    "cigemm_linear_f32": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _ci, _vp, _i64]),
     "cigemm_fill_random_f32": (_ci, [_vp, _vp, _i64, _u64, _f32, _f32]),
     "cigemm_fill_random_bf16": (_ci, [_vp, _vp, _i64, _u64, _f32, _f32]),
     "cigemm_fill_random_f16": (_ci, [_vp, _vp, _i64, _u64, _f32, _f32]),
@@ -172,6 +174,21 @@ class Handle:
         torch = _torch()
         assert A.dtype == torch.float32 and B.dtype == torch.float32
         return self._gemm("cigemm_gemm_f32", A, B, out, torch.float32)
+
+    def linear_f32(self, X, W, bias=None, act=ACT_NONE, out=None):
+        """out = act(bias + X @ W) with W stored K x N (input-major)."""
+        torch = _torch()
+        assert X.dtype == torch.float32 and W.dtype == torch.float32
+        M, K = X.shape
+        K2, N = W.shape
+        assert K == K2 and (bias is None or (bias.dtype == torch.float32 and bias.numel() == N))
+        if out is None:
+            out = torch.empty((M, N), dtype=torch.float32, device=X.device)
+        st = self.lib.cigemm_linear_f32(self._h, M, N, K, X.data_ptr(), self._ld(X), W.data_ptr(),
+                                        self._ld(W), bias.data_ptr() if bias is not None else None,
+                                        act, out.data_ptr(), self._ld(out))
+        self._check(st, "cigemm_linear_f32")
+        return out
 
     def gemm_f16(self, A, B, out=None):
         torch = _torch()

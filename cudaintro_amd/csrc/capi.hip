@@ -155,6 +155,20 @@ cigemmStatus_t cigemm_gemm_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K
   return check_launch(h, "cigemm_gemm_f32");
 }
 
+cigemmStatus_t cigemm_linear_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K, const float* X,
+                                 int64_t ldx, const float* W, int64_t ldw, const float* bias,
+                                 cigemmActivation_t act, float* out, int64_t ldo) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if (act != CIGEMM_ACT_NONE && act != CIGEMM_ACT_RELU)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "cigemm_linear_f32: bad activation %d", (int)act);
+  cigemmStatus_t st = check_gemm_args(h, "cigemm_linear_f32", M, N, K, X, ldx, W, ldw, N, out, ldo);
+  if (st != CIGEMM_STATUS_SUCCESS || M == 0 || N == 0) return st;
+  BiasAct ba{bias, act == CIGEMM_ACT_RELU};
+  if (!launch_f32_mfma(h, M, N, K, X, ldx, W, ldw, out, ldo, &ba))
+    launch_generic_f32(h, M, N, K, X, ldx, W, ldw, out, ldo, &ba);
+  return check_launch(h, "cigemm_linear_f32");
+}
+
 static cigemmStatus_t gemm16(cigemmHandle_t h, const char* name, bool bf16, int64_t M, int64_t N,
                              int64_t K, const uint16_t* A, int64_t lda, const uint16_t* B,
                              int64_t ldb, uint16_t* C, int64_t ldc) {

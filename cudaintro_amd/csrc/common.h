@@ -79,6 +79,18 @@ struct F16 {
 // ---- epilogues --------------------------------------------------------------------------
 // Each epilogue stores one accumulator for output element (row, col).
 
+struct EpiBiasActF32 {  // fp32 linear layer: act(acc + bias[col])
+  float* C;
+  int64_t ldc;
+  const float* bias;
+  int relu;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float acc) const {
+    float v = bias ? __fadd_rn(acc, bias[c]) : acc;
+    if (relu) v = fmaxf(0.0f, v);
+    C[r * ldc + c] = v;
+  }
+};
+
 struct EpiStoreF32 {  // fp32 GEMM
   float* C;
   int64_t ldc;
@@ -128,6 +140,12 @@ struct EpiDequant {
   }
 };
 
+// Bias + activation of the linear-layer entry point (bias may be null).
+struct BiasAct {
+  const float* bias;
+  int relu;
+};
+
 struct DequantArgs {
   const float* sa;
   const float* sb;
@@ -147,7 +165,8 @@ struct DequantArgs {
 
 // gemm_generic.hip: any shape, any alignment.
 void launch_generic_f32(cigemmContext*, int64_t M, int64_t N, int64_t K, const float* A,
-                        int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc);
+                        int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                        const BiasAct* ba = nullptr);
 void launch_generic_16(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
                        const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                        uint16_t* C, int64_t ldc);
@@ -157,7 +176,8 @@ void launch_generic_i8(cigemmContext*, int64_t M, int64_t N, int64_t K, const in
 
 // gemm_f32.hip
 bool launch_f32_mfma(cigemmContext*, int64_t M, int64_t N, int64_t K, const float* A,
-                     int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc);
+                     int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                     const BiasAct* ba = nullptr);
 // gemm_16b.hip
 bool launch_16b_mfma(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
                      const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,

@@ -57,6 +57,40 @@ struct EpiStoreF32x4 {
   EpiStoreF32x4 shift_cols(int64_t c0) const { return EpiStoreF32x4{C + c0, ldc}; }
 };
 
+// fp32 linear layer: act(acc + bias[col]); RELU and HAS_BIAS are compile-time.
+template <bool HAS_BIAS, bool RELU>
+struct EpiBiasActF32x4 {
+  float* C;
+  int64_t ldc;
+  const float* bias;
+  static constexpr int OUT_BYTES = 4;
+  __device__ __forceinline__ u32x4 pack(int64_t, int64_t c, float v0, float v1, float v2,
+                                        float v3) const {
+    f32x4 v = {v0, v1, v2, v3};
+    if (HAS_BIAS) {
+      const f32x4 b = *reinterpret_cast<const f32x4*>(bias + c);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = __fadd_rn(v[e], b[e]);
+    }
+    if (RELU) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = fmaxf(0.0f, v[e]);
+    }
+    return __builtin_bit_cast(u32x4, v);
+  }
+  __device__ __forceinline__ char* out_row(int64_t r) const {
+    return reinterpret_cast<char*>(C + r * ldc);
+  }
+  __device__ __forceinline__ void side(int64_t, int64_t, float, float, float, float) const {}
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float v0, float v1, float v2,
+                                             float v3) const {
+    *reinterpret_cast<u32x4*>(C + r * ldc + c) = pack(r, c, v0, v1, v2, v3);
+  }
+  EpiBiasActF32x4 shift_cols(int64_t c0) const {
+    return EpiBiasActF32x4{C + c0, ldc, HAS_BIAS ? bias + c0 : bias};
+  }
+};
+
 struct EpiStoreI32x4 {
   int32_t* C;
   int64_t ldc;

@@ -120,7 +120,15 @@ inline dim3 generic_grid(int64_t M, int64_t N) {
 }  // namespace
 
 void launch_generic_f32(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const float* A,
-                        int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc) {
+                        int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                        const BiasAct* ba) {
+  if (ba) {
+    EpiBiasActF32 epi{C, ldc, ba->bias, ba->relu};
+    hipLaunchKernelGGL((gemm_generic_kernel<float, LoadF32, MacF32, false, EpiBiasActF32>),
+                       generic_grid(M, N), dim3(256), 0, ctx->stream, M, N, K, A, lda, B, ldb, epi);
+    ctx->last_kernel = "f32_generic_64x64x16_bias_act";
+    return;
+  }
   EpiStoreF32 epi{C, ldc};
   hipLaunchKernelGGL((gemm_generic_kernel<float, LoadF32, MacF32, false, EpiStoreF32>),
                      generic_grid(M, N), dim3(256), 0, ctx->stream, M, N, K, A, lda, B, ldb, epi);

@@ -138,6 +138,23 @@ CIGEMM_API cigemmStatus_t cigemm_gemm_i8_dequant(
     cigemmScaleMode_t scaleA_mode, const float* scaleB, cigemmScaleMode_t scaleB_mode,
     void* out, cigemmOutType_t out_type, int64_t ldo, int32_t* acc_out, int64_t ldacc);
 
+/* ---- linear layer: GEMM with bias and activation fused ------------------------------ */
+
+typedef enum cigemmActivation {
+  CIGEMM_ACT_NONE = 0,
+  CIGEMM_ACT_RELU = 1 /* max(0, x) */
+} cigemmActivation_t;
+
+/* out[M x N] = act(bias[j] + X[M x K] . W[K x N]), fp32, row-major.  Replaces the MLP forward
+ * kernels of the reference's MNIST demo -- forwardInputToHiddenKernel followed by
+ * reluActivationKernel (MNIST/mnist_nn.cu:10-24, 27-33; 20000 x 784 x 512) and
+ * forwardHiddenToOutputKernel (MNIST/mnist_nn.cu:36-49; 20000 x 512 x 10) -- which are
+ * exactly this with W stored input-major (W[i * N + j]).  `bias` has N entries (NULL = none). */
+CIGEMM_API cigemmStatus_t cigemm_linear_f32(cigemmHandle_t handle, int64_t M, int64_t N,
+                                            int64_t K, const float* X, int64_t ldx,
+                                            const float* W, int64_t ldw, const float* bias,
+                                            cigemmActivation_t act, float* out, int64_t ldo);
+
 /* ---- device-side input generation -------------------------------------------------- */
 
 /* Replace fill_random_fp32 / _bf16 / _fp16 / _int8 (quantization/GEMM_fp32.cu:7-17,

@@ -54,6 +54,7 @@ def _load():
         "oracle_dequant_bf16": (None, [i64, i64, vp, i64, vp, ci, vp, ci, vp, i64]),
         "oracle_quantize_rows_i8": (None, [i64, i64, vp, i64, vp, i64, vp]),
         "oracle_checkResult": (i64, [vp, vp, ci, f32, ci]),
+        "oracle_linear_f32": (None, [i64, i64, i64, vp, vp, vp, ci, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -206,12 +207,6 @@ def gemm_i8_i64_ijk(A, B, b_is_nk=False):
 
 
 # ---- epilogue / quantizer / compare ---------------------------------------------------
-def _scales(s, n):
-    s = _c(np.atleast_1d(s), np.float32)
-    assert s.size in (1, n)
-    return s, int(s.size == n and n != 1) if s.size != 1 else 0
-
-
 def dequant(acc, sa, sb, out_dtype="f32", sa_per_row=None, sb_per_col=None):
     acc = _c(acc, np.int32)
     M, N = acc.shape
@@ -240,6 +235,19 @@ def quantize_rows_i8(x):
     s = np.empty(rows, np.float32)
     lib.oracle_quantize_rows_i8(rows, cols, _p(x), cols, _p(q), cols, _p(s))
     return q, s
+
+
+def linear_f32(X, W, bias=None, relu=False):
+    """MNIST MLP forward layer (MNIST/mnist_nn.cu:10-24, 27-33, 36-49)."""
+    X = _c(X, np.float32)
+    W = _c(W, np.float32)
+    M, K = X.shape
+    N = W.shape[1]
+    assert W.shape[0] == K
+    b = _c(bias, np.float32) if bias is not None else None
+    out = np.empty((M, N), np.float32)
+    lib.oracle_linear_f32(M, N, K, _p(X), _p(W), _p(b) if b is not None else None, int(relu), _p(out))
+    return out
 
 
 def checkResult(gpu, cpu, eps=1e-5, verbose=False):

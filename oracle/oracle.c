@@ -21,6 +21,8 @@
  *                                          raw int32: quantization/GEMM_int8.cu:48-56);
  *                                          pinned against numpy float32 arithmetic.
  *   oracle_quantize_rows_i8                build-defined; pinned by hand cases.
+ *   oracle_linear_f32                      MNIST MLP forward layer; pinned by bias-only,
+ *                                          identity-weight and ReLU sign cases and numpy.
  *   cuBLAS's own summation order           parity unpinned: closed source, absent, and the
  *                                          reference holds no output for it.
  *
@@ -343,6 +345,27 @@ ORACLE_API void oracle_quantize_rows_i8(int64_t rows, int64_t cols, const float*
       if (r < -127.0f) r = -127.0f;
       q[i * ldq + j] = (int8_t)r;
     }
+  }
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* MLP forward layer of the MNIST demo: MNIST/mnist_nn.cu:10-24 (input -> hidden),       */
+/* 27-33 (ReLU), 36-49 (hidden -> output).  sum starts at the bias and adds the products */
+/* one at a time in ascending i; W is input-major (W[i * N + j]).                        */
+/* ------------------------------------------------------------------------------------ */
+ORACLE_API void oracle_linear_f32(int64_t M, int64_t N, int64_t K, const float* X, const float* W,
+                                  const float* bias, int relu, float* out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t b = 0; b < M; ++b) {
+    float* o = out + b * N;
+    for (int64_t j = 0; j < N; ++j) o[j] = bias ? bias[j] : 0.0f;
+    for (int64_t i = 0; i < K; ++i) {
+      const float x = X[b * K + i];
+      const float* w = W + i * N;
+      for (int64_t j = 0; j < N; ++j) o[j] += x * w[j];
+    }
+    if (relu)
+      for (int64_t j = 0; j < N; ++j) o[j] = fmaxf(0.0f, o[j]);
   }
 }
 
