@@ -9,6 +9,11 @@ library and a gfx950 device.
 from .cigemm import (  # noqa: F401
     ACT_NONE,
     ACT_RELU,
+    ALGO_DEFAULT,
+    ALGO_GENERIC,
+    ALGO_SKINNY,
+    ALGO_SMALL,
+    ALGO_TILE,
     B_KN,
     B_NK,
     OUT_BF16,

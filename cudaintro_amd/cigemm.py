@@ -17,6 +17,7 @@ _SUITE = os.path.join(_HERE, "gemm_suite")
 
 B_KN, B_NK = 0, 1
 ACT_NONE, ACT_RELU = 0, 1
+ALGO_DEFAULT, ALGO_GENERIC, ALGO_TILE, ALGO_SKINNY, ALGO_SMALL = -1, 0, 1, 2, 3
 SCALE_TENSOR, SCALE_VECTOR = 0, 1
 OUT_F32, OUT_BF16 = 0, 1
 
@@ -67,6 +68,8 @@ SIGNATURES = {
     "cigemmGetLastErrorString": (C.c_char_p, [_vp]),
     "cigemmGetVersion": (_ci, []),
     "cigemmGetLastKernelName": (C.c_char_p, [_vp]),
+    "cigemmSetAlgo": (C.c_int, [_vp, C.c_int]),
+    "cigemmGetAlgo": (C.c_int, [_vp, C.POINTER(C.c_int)]),
     "cigemm_gemm_f32": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "cigemm_gemm_f16": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "cigemm_gemm_bf16": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
@@ -143,6 +146,30 @@ class Handle:
 
     def set_stream(self, raw_stream: int):
         self._check(self.lib.cigemmSetStream(self._h, _vp(raw_stream)), "cigemmSetStream")
+
+    def set_algo(self, algo: int):
+        """Restrict following GEMM calls to one kernel family (``ALGO_*``)."""
+        self._check(self.lib.cigemmSetAlgo(self._h, algo), "cigemmSetAlgo")
+
+    def get_algo(self) -> int:
+        v = C.c_int(0)
+        self._check(self.lib.cigemmGetAlgo(self._h, C.byref(v)), "cigemmGetAlgo")
+        return v.value
+
+    def algo(self, algo: int):
+        """Context manager: ``with h.algo(ALGO_TILE): ...`` and back to the previous choice."""
+        import contextlib
+
+        @contextlib.contextmanager
+        def scope():
+            prev = self.get_algo()
+            self.set_algo(algo)
+            try:
+                yield self
+            finally:
+                self.set_algo(prev)
+
+        return scope()
 
     @property
     def raw(self):

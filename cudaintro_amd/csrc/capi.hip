@@ -88,6 +88,7 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->num_cus = prop.multiProcessorCount;
   ctx->stream = nullptr;
   ctx->last_kernel = "";
+  ctx->algo = CIGEMM_ALGO_DEFAULT;
   ctx->last_error[0] = '\0';
   ctx->ws_partial_bytes = (size_t)16 << 20;
   ctx->ws_counter_bytes = (size_t)64 << 10;
@@ -145,13 +146,57 @@ int cigemmGetVersion(void) { return 100; }
 
 const char* cigemmGetLastKernelName(cigemmHandle_t h) { return valid(h) ? h->last_kernel : ""; }
 
+cigemmStatus_t cigemmSetAlgo(cigemmHandle_t h, cigemmAlgo_t algo) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if ((int)algo < CIGEMM_ALGO_DEFAULT || (int)algo > CIGEMM_ALGO_SMALL)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "cigemmSetAlgo: bad algo %d", (int)algo);
+  h->algo = (int)algo;
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+cigemmStatus_t cigemmGetAlgo(cigemmHandle_t h, cigemmAlgo_t* algo) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if (!algo) return fail(h, CIGEMM_STATUS_INVALID_VALUE, "cigemmGetAlgo: null pointer");
+  *algo = (cigemmAlgo_t)h->algo;
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+static cigemmStatus_t algo_refused(cigemmHandle_t h, const char* name) {
+  return fail(h, CIGEMM_STATUS_NOT_SUPPORTED,
+              "%s: the selected kernel family (algo %d) does not take this call", name, h->algo);
+}
+
+// fp32 dispatch.  DEFAULT: one of the two MFMA kernels when the shape allows, else the
+// any-shape kernel.  Returns false when a selected family refuses the call.
+static bool dispatch_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K, const float* A,
+                         int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                         const BiasAct* ba) {
+  switch (h->algo) {
+    case CIGEMM_ALGO_TILE:
+      return launch_f32_tile(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
+    case CIGEMM_ALGO_SMALL:
+      if (!f32_small_shape_ok(M, N, K, A, lda)) return false;
+      launch_f32_small(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
+      return true;
+    case CIGEMM_ALGO_SKINNY:
+      return false;
+    case CIGEMM_ALGO_GENERIC:
+      launch_generic_f32(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
+      return true;
+    default:
+      if (!launch_f32_mfma(h, M, N, K, A, lda, B, ldb, C, ldc, ba))
+        launch_generic_f32(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
+      return true;
+  }
+}
+
 cigemmStatus_t cigemm_gemm_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K, const float* A,
                                int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc) {
   if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
   cigemmStatus_t st = check_gemm_args(h, "cigemm_gemm_f32", M, N, K, A, lda, B, ldb, N, C, ldc);
   if (st != CIGEMM_STATUS_SUCCESS || M == 0 || N == 0) return st;
-  if (!launch_f32_mfma(h, M, N, K, A, lda, B, ldb, C, ldc))
-    launch_generic_f32(h, M, N, K, A, lda, B, ldb, C, ldc);
+  if (!dispatch_f32(h, M, N, K, A, lda, B, ldb, C, ldc, nullptr))
+    return algo_refused(h, "cigemm_gemm_f32");
   return check_launch(h, "cigemm_gemm_f32");
 }
 
@@ -164,8 +209,8 @@ cigemmStatus_t cigemm_linear_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t
   cigemmStatus_t st = check_gemm_args(h, "cigemm_linear_f32", M, N, K, X, ldx, W, ldw, N, out, ldo);
   if (st != CIGEMM_STATUS_SUCCESS || M == 0 || N == 0) return st;
   BiasAct ba{bias, act == CIGEMM_ACT_RELU};
-  if (!launch_f32_mfma(h, M, N, K, X, ldx, W, ldw, out, ldo, &ba))
-    launch_generic_f32(h, M, N, K, X, ldx, W, ldw, out, ldo, &ba);
+  if (!dispatch_f32(h, M, N, K, X, ldx, W, ldw, out, ldo, &ba))
+    return algo_refused(h, "cigemm_linear_f32");
   return check_launch(h, "cigemm_linear_f32");
 }
 
@@ -175,10 +220,19 @@ static cigemmStatus_t gemm16(cigemmHandle_t h, const char* name, bool bf16, int6
   if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
   cigemmStatus_t st = check_gemm_args(h, name, M, N, K, A, lda, B, ldb, N, C, ldc);
   if (st != CIGEMM_STATUS_SUCCESS || M == 0 || N == 0) return st;
-  // decode shapes (M <= 32) first: they are bandwidth problems with their own kernel
-  if (!launch_skinny_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc) &&
-      !launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc))
-    launch_generic_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc);
+  bool ok = true;
+  switch (h->algo) {
+    case CIGEMM_ALGO_SKINNY: ok = launch_skinny_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
+    case CIGEMM_ALGO_TILE: ok = launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
+    case CIGEMM_ALGO_SMALL: ok = false; break;
+    case CIGEMM_ALGO_GENERIC: launch_generic_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
+    default:
+      // decode shapes (M <= 32) first: they are bandwidth problems with their own kernel
+      if (!launch_skinny_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc) &&
+          !launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc))
+        launch_generic_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc);
+  }
+  if (!ok) return algo_refused(h, name);
   return check_launch(h, name);
 }
 
@@ -199,9 +253,18 @@ static cigemmStatus_t gemm_i8(cigemmHandle_t h, const char* name, int64_t M, int
                               cigemmBLayout_t b_layout, int32_t* C, int64_t ldc,
                               const DequantArgs* dq) {
   const bool b_nk = b_layout == CIGEMM_B_NK;
-  if (!launch_skinny_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq) &&
-      !launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq))
-    launch_generic_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);
+  bool ok = true;
+  switch (h->algo) {
+    case CIGEMM_ALGO_SKINNY: ok = launch_skinny_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq); break;
+    case CIGEMM_ALGO_TILE: ok = launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq); break;
+    case CIGEMM_ALGO_SMALL: ok = false; break;
+    case CIGEMM_ALGO_GENERIC: launch_generic_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq); break;
+    default:
+      if (!launch_skinny_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq) &&
+          !launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq))
+        launch_generic_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);
+  }
+  if (!ok) return algo_refused(h, name);
   return check_launch(h, name);
 }
 

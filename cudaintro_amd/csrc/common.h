@@ -16,6 +16,7 @@ struct cigemmContext {
   int num_cus;
   hipStream_t stream;
   const char* last_kernel;
+  int algo;  // cigemmAlgo_t; -1 = choose by shape
   // Device scratch of the split-K kernels, allocated once at create: `ws_partial_bytes` of
   // partial sums followed by `ws_counter_bytes` of arrival counters (zero between calls).
   void* workspace;
@@ -174,10 +175,20 @@ void launch_generic_i8(cigemmContext*, int64_t M, int64_t N, int64_t K, const in
                        int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
                        int64_t ldc, const DequantArgs* dq);
 
-// gemm_f32.hip
+// gemm_f32.hip: launch_f32_tile takes what the LDS-tiled kernel takes; launch_f32_mfma
+// chooses between it and the small-tile kernel.  Both return false without launching when
+// the shape is not theirs.
+bool launch_f32_tile(cigemmContext*, int64_t M, int64_t N, int64_t K, const float* A,
+                     int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                     const BiasAct* ba = nullptr);
 bool launch_f32_mfma(cigemmContext*, int64_t M, int64_t N, int64_t K, const float* A,
                      int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
                      const BiasAct* ba = nullptr);
+// gemm_f32_small.hip: 32x32 tile per workgroup, k split over the waves.
+bool f32_small_shape_ok(int64_t M, int64_t N, int64_t K, const float* A, int64_t lda);
+void launch_f32_small(cigemmContext*, int64_t M, int64_t N, int64_t K, const float* A,
+                      int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                      const BiasAct* ba = nullptr);
 // gemm_16b.hip
 bool launch_16b_mfma(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
                      const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,

@@ -1,0 +1,120 @@
+// fp32 GEMM for problems too small (or too narrow) to fill the chip with 256-column tiles:
+// one 32x32 output tile per 256-lane workgroup, the k range split over the four waves
+// (each wave: v_mfma_f32_32x32x2_f32 on operands loaded straight from global memory into
+// registers, no LDS staging), the four partial tiles summed through LDS in wave order
+// (deterministic), then bias / activation and the store.  512^3 gives 256 workgroups
+// instead of the 16 of the 64x256 tile; an N = 10 output layer
+// (MNIST/mnist_nn.cu:36-49) streams its activations once with row-clamped loads.
+//
+// Ragged M and N: loads past the edge re-read the last valid row / column, stores are
+// masked.  K must be a multiple of 8 and A's rows 16-byte aligned.
+#include "common.h"
+
+namespace cig {
+namespace {
+
+constexpr int ST = 32;        // tile edge = one MFMA tile
+constexpr int RED_LD = 36;    // floats per row of a partial tile in LDS (16-byte rows, padded)
+
+template <bool HAS_BIAS, bool RELU>
+__global__ __launch_bounds__(256) void f32_small_kernel(int M, int N, int K, int tiles_n,
+                                                        const float* __restrict__ A, int64_t lda,
+                                                        const float* __restrict__ B, int64_t ldb,
+                                                        float* __restrict__ C, int64_t ldc,
+                                                        const float* __restrict__ bias) {
+  __shared__ __attribute__((aligned(16))) float red[4][ST][RED_LD];
+  const int t = threadIdx.x;
+  const int w = t >> 6, l = t & 63;
+  const int r = l & 31, h = l >> 5;
+  const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+  const int m0 = tm * ST, n0 = tn * ST;
+
+  // Lane (r, h) feeds row m0+r of A and column n0+r of B at k = kb + 4h + e, e = 0..3,
+  // for every 8-deep block kb of its wave's share of K.
+  const int row = min(m0 + r, M - 1);
+  const int col = min(n0 + r, N - 1);
+  const int nblk = K >> 3;
+  const int b0 = (int)((int64_t)w * nblk / 4), b1 = (int)((int64_t)(w + 1) * nblk / 4);
+  const float* ap = A + (int64_t)row * lda + 4 * h + 8 * (int64_t)b0;
+  const float* bp = B + (4 * h + 8 * (int64_t)b0) * ldb + col;
+
+  f32x16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+
+#pragma unroll 4
+  for (int b = b0; b < b1; ++b) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(ap);
+    const float x0 = bp[0], x1 = bp[ldb], x2 = bp[2 * ldb], x3 = bp[3 * ldb];
+    // (B fragment, A fragment): the lane then holds four consecutive columns of one row.
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x0, a[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1, a[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x2, a[2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x3, a[3], acc, 0, 0, 0);
+    ap += 8;
+    bp += 8 * ldb;
+  }
+
+  // acc[4q+e] is C[m0 + r][n0 + 8q + 4h + e].
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const f32x4 v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+    *reinterpret_cast<f32x4*>(&red[w][r][8 * q + 4 * h]) = v;
+  }
+  __syncthreads();
+
+  const int om = t >> 3, on = (t & 7) * 4;
+  f32x4 s = *reinterpret_cast<const f32x4*>(&red[0][om][on]);
+#pragma unroll
+  for (int ww = 1; ww < 4; ++ww) {
+    const f32x4 p = *reinterpret_cast<const f32x4*>(&red[ww][om][on]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] = __fadd_rn(s[e], p[e]);
+  }
+  const int gm = m0 + om, gn = n0 + on;
+  if (gm >= M) return;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (HAS_BIAS) s[e] = __fadd_rn(s[e], bias[min(gn + e, N - 1)]);
+    if (RELU) s[e] = fmaxf(0.0f, s[e]);
+  }
+  float* out = C + (int64_t)gm * ldc + gn;
+  if (gn + 3 < N && ((reinterpret_cast<uintptr_t>(out) & 15) == 0)) {
+    *reinterpret_cast<f32x4*>(out) = s;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (gn + e < N) out[e] = s[e];
+  }
+}
+
+}  // namespace
+
+bool f32_small_shape_ok(int64_t M, int64_t N, int64_t K, const float* A, int64_t lda) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 8) return false;
+  if (lda % 4 || (reinterpret_cast<uintptr_t>(A) & 15)) return false;
+  if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return false;
+  const int64_t tiles = ((M + ST - 1) / ST) * ((N + ST - 1) / ST);
+  return tiles <= 0x7fffffff;
+}
+
+void launch_f32_small(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const float* A,
+                      int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                      const BiasAct* ba) {
+  const int tiles_m = (int)((M + ST - 1) / ST), tiles_n = (int)((N + ST - 1) / ST);
+  const dim3 grid((unsigned)(tiles_m * (int64_t)tiles_n)), block(256);
+  const float* bias = ba ? ba->bias : nullptr;
+  const bool relu = ba && ba->relu;
+#define CIG_SMALL(HB, RL)                                                                   \
+  hipLaunchKernelGGL((f32_small_kernel<HB, RL>), grid, block, 0, ctx->stream, (int)M, (int)N, \
+                     (int)K, tiles_n, A, lda, B, ldb, C, ldc, bias)
+  if (bias) {
+    if (relu) CIG_SMALL(true, true); else CIG_SMALL(true, false);
+  } else {
+    if (relu) CIG_SMALL(false, true); else CIG_SMALL(false, false);
+  }
+#undef CIG_SMALL
+  ctx->last_kernel = ba ? "f32_mfma_small_32x32_ksplit4_bias_act" : "f32_mfma_small_32x32_ksplit4";
+}
+
+}  // namespace cig

@@ -91,8 +91,23 @@ CIGEMM_API const char* cigemmGetLastErrorString(cigemmHandle_t handle);
 CIGEMM_API int cigemmGetVersion(void);
 
 /* Name of the kernel family the last successful GEMM call on this handle dispatched to
- * (for tests and profiles), e.g. "bf16_mfma_256x256x64". */
+ * (for tests and profiles), e.g. "bf16_mfma_256x256x32_ring4". */
 CIGEMM_API const char* cigemmGetLastKernelName(cigemmHandle_t handle);
+
+/* Kernel family selection: the counterpart of cublasGemmEx's `algo` argument (the reference
+ * passes CUBLAS_GEMM_DEFAULT_TENSOR_OP, quantization/GEMM_bf16.cu:56), kept on the handle.
+ * DEFAULT lets the library choose by shape.  A specific family restricts every following GEMM
+ * call on the handle to it; a call whose shape, alignment or type that family does not take
+ * returns CIGEMM_STATUS_NOT_SUPPORTED and launches nothing. */
+typedef enum cigemmAlgo {
+  CIGEMM_ALGO_DEFAULT = -1,
+  CIGEMM_ALGO_GENERIC = 0, /* any-shape scalar kernel (fp32: bit-exact with the CPU loop) */
+  CIGEMM_ALGO_TILE = 1,    /* LDS-tiled MFMA kernel, 256-column tiles */
+  CIGEMM_ALGO_SKINNY = 2,  /* M <= 32 split-K streaming kernel (16-bit K x N, int8 N x K) */
+  CIGEMM_ALGO_SMALL = 3    /* fp32 32x32 tile per workgroup, k split over the waves */
+} cigemmAlgo_t;
+CIGEMM_API cigemmStatus_t cigemmSetAlgo(cigemmHandle_t handle, cigemmAlgo_t algo);
+CIGEMM_API cigemmStatus_t cigemmGetAlgo(cigemmHandle_t handle, cigemmAlgo_t* algo);
 
 /* ---- GEMM: C[M x N] = A[M x K] . B[K x N], row-major ------------------------------- */
 

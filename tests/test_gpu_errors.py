@@ -60,3 +60,43 @@ def test_destroyed_handle_is_rejected(torch_gpu):
     s.synchronize()
     assert (c.cpu().numpy() == 64).all()
     h2.close()
+
+
+def test_kernel_family_selection(torch_gpu):
+    """cigemmSetAlgo restricts the dispatch; a family that does not take the call refuses it
+    with NOT_SUPPORTED, writes nothing, and the handle keeps working."""
+    torch = torch_gpu
+    h = ci.Handle()
+    assert h.get_algo() == ci.ALGO_DEFAULT
+    assert h.lib.cigemmSetAlgo(h.raw, 4) == Status.INVALID_VALUE
+    assert h.lib.cigemmSetAlgo(h.raw, -2) == Status.INVALID_VALUE
+    assert h.lib.cigemmGetAlgo(h.raw, None) == Status.INVALID_VALUE
+    a = torch.ones((64, 64), dtype=torch.float32, device="cuda")
+    out = torch.full((64, 64), 5.0, dtype=torch.float32, device="cuda")
+    for algo in (ci.ALGO_SKINNY,):                       # no fp32 skinny kernel
+        h.set_algo(algo)
+        with pytest.raises(ci.CigemmError, match="NOT_SUPPORTED"):
+            h.gemm_f32(a, a, out=out)
+    odd = torch.ones((64, 63), dtype=torch.float32, device="cuda")    # K = 63
+    for algo in (ci.ALGO_TILE, ci.ALGO_SMALL):
+        h.set_algo(algo)
+        with pytest.raises(ci.CigemmError, match="NOT_SUPPORTED"):
+            h.gemm_f32(odd, torch.ones((63, 64), device="cuda"), out=out)
+    a16 = torch.ones((64, 64), dtype=torch.bfloat16, device="cuda")
+    a8 = torch.ones((64, 64), dtype=torch.int8, device="cuda")
+    for algo in (ci.ALGO_SKINNY, ci.ALGO_SMALL):         # M = 64 is not a skinny shape
+        h.set_algo(algo)
+        with pytest.raises(ci.CigemmError, match="NOT_SUPPORTED"):
+            h.gemm_bf16(a16, a16)
+        with pytest.raises(ci.CigemmError, match="NOT_SUPPORTED"):
+            h.gemm_i8_i32(a8, a8)
+    torch.cuda.synchronize()
+    assert (out.cpu().numpy() == 5.0).all()
+    for algo, frag in ((ci.ALGO_GENERIC, "generic"), (ci.ALGO_TILE, "mfma_256"), (ci.ALGO_DEFAULT, "mfma")):
+        h.set_algo(algo)
+        c = h.gemm_bf16(a16, a16)
+        assert frag in h.last_kernel
+        assert (c.float().cpu().numpy() == 64.0).all()
+        c = h.gemm_i8_i32(a8, a8)
+        assert (c.cpu().numpy() == 64).all()
+    h.close()

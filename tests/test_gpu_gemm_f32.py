@@ -2,6 +2,7 @@
 import numpy as np
 import pytest
 
+import cudaintro_amd as ci
 from cudaintro_amd import workloads as wl
 
 pytestmark = pytest.mark.gpu
@@ -94,48 +95,98 @@ def test_k_zero_and_empty(handle, torch_gpu):
                     torch.empty((3, 5), dtype=torch.float32, device="cuda"))
 
 
-def test_mfma_path_onehot_and_bound(handle, torch_gpu, oracle, rng):
-    """The fp32 MFMA tile kernel: one-hot rows/columns select exactly, random inputs stay within
+MFMA_ALGOS = [pytest.param(ci.ALGO_TILE, id="tile"), pytest.param(ci.ALGO_SMALL, id="small")]
+
+
+@pytest.mark.parametrize("algo", MFMA_ALGOS)
+def test_mfma_path_onehot_and_bound(handle, torch_gpu, oracle, rng, algo):
+    """Both fp32 MFMA kernels: one-hot rows/columns select exactly, random inputs stay within
     the fp32 summation bound of fp64, leading dimensions and guard columns are respected."""
     torch = torch_gpu
     M, N, K = 512, 768, 272
-    Bf = rng.normal(size=(K, N)).astype(np.float32)
-    perm = rng.integers(0, K, size=M)
-    A = np.zeros((M, K), np.float32)
-    A[np.arange(M), perm] = 1.0
-    C = run(handle, torch, A, Bf)
-    assert "mfma" in handle.last_kernel, handle.last_kernel
-    np.testing.assert_array_equal(C, Bf[perm])
-    Af = rng.normal(size=(M, K)).astype(np.float32)
-    permn = rng.integers(0, K, size=N)
-    B = np.zeros((K, N), np.float32)
-    B[permn, np.arange(N)] = 1.0
-    np.testing.assert_array_equal(run(handle, torch, Af, B), Af[:, permn])
-    # sub-blocks of larger buffers
-    bigA = torch.from_numpy(rng.normal(size=(M, K + 40)).astype(np.float32)).cuda()
-    bigB = torch.from_numpy(rng.normal(size=(K, N + 12)).astype(np.float32)).cuda()
-    out = torch.full((M, N + 8), -3.0, dtype=torch.float32, device="cuda")
-    a, b, c = bigA[:, 8:8 + K], bigB[:, 4:4 + N], out[:, 4:4 + N]
-    handle.gemm_f32(a, b, out=c)
-    assert "mfma" in handle.last_kernel
+    with handle.algo(algo):
+        Bf = rng.normal(size=(K, N)).astype(np.float32)
+        perm = rng.integers(0, K, size=M)
+        A = np.zeros((M, K), np.float32)
+        A[np.arange(M), perm] = 1.0
+        C = run(handle, torch, A, Bf)
+        assert ("small" in handle.last_kernel) == (algo == ci.ALGO_SMALL), handle.last_kernel
+        assert "mfma" in handle.last_kernel
+        np.testing.assert_array_equal(C, Bf[perm])
+        Af = rng.normal(size=(M, K)).astype(np.float32)
+        permn = rng.integers(0, K, size=N)
+        B = np.zeros((K, N), np.float32)
+        B[permn, np.arange(N)] = 1.0
+        np.testing.assert_array_equal(run(handle, torch, Af, B), Af[:, permn])
+        # sub-blocks of larger buffers
+        bigA = torch.from_numpy(rng.normal(size=(M, K + 40)).astype(np.float32)).cuda()
+        bigB = torch.from_numpy(rng.normal(size=(K, N + 12)).astype(np.float32)).cuda()
+        out = torch.full((M, N + 8), -3.0, dtype=torch.float32, device="cuda")
+        a, b, c = bigA[:, 8:8 + K], bigB[:, 4:4 + N], out[:, 4:4 + N]
+        handle.gemm_f32(a, b, out=c)
+        assert "mfma" in handle.last_kernel
     ref, S = oracle.gemm_f64(a.cpu().numpy(), b.cpu().numpy(), with_abs=True)
     assert (np.abs(c.cpu().numpy() - ref) <= K * 2.0 ** -24 * S).all()
     o = out.cpu().numpy()
     assert (o[:, :4] == -3.0).all() and (o[:, 4 + N:] == -3.0).all()
 
 
-@pytest.mark.parametrize("shape", [(33, 4, 16), (100, 260, 48), (257, 1028, 64), (20000, 512, 784), (1000, 12, 512)])
-def test_mfma_path_ragged_shapes(handle, torch_gpu, oracle, rng, shape):
-    """Any M, N a multiple of 4, K a multiple of 16 go through the MFMA tile kernel with
-    clamped loads and masked stores; guard rows/columns of the output stay untouched."""
-    torch = torch_gpu
+def ragged_check(handle, torch, oracle, rng, algo, shape, pad_cols=4):
     M, N, K = shape
     A = rng.uniform(-1, 1, size=(M, K)).astype(np.float32)
     B = rng.uniform(-1, 1, size=(K, N)).astype(np.float32)
-    out = torch.full((M + 3, N + 4), -9.0, dtype=torch.float32, device="cuda")
-    handle.gemm_f32(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), out=out[:M, :N])
-    assert "mfma" in handle.last_kernel, handle.last_kernel
+    out = torch.full((M + 3, N + pad_cols), -9.0, dtype=torch.float32, device="cuda")
+    with handle.algo(algo):
+        handle.gemm_f32(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), out=out[:M, :N])
+        name = handle.last_kernel
     o = out.cpu().numpy()
     ref, S = oracle.gemm_f64(A, B, with_abs=True)
     assert (np.abs(o[:M, :N] - ref) <= K * 2.0 ** -24 * S + 1e-30).all()
     assert (o[M:] == -9.0).all() and (o[:, N:] == -9.0).all()
+    return name
+
+
+@pytest.mark.parametrize("shape", [(33, 4, 16), (100, 260, 48), (257, 1028, 64), (20000, 512, 784), (1000, 12, 512)])
+def test_tile_kernel_ragged_shapes(handle, torch_gpu, oracle, rng, shape):
+    """Any M, N a multiple of 4, K a multiple of 16 go through the MFMA tile kernel with
+    clamped loads and masked stores; guard rows/columns of the output stay untouched."""
+    name = ragged_check(handle, torch_gpu, oracle, rng, ci.ALGO_TILE, shape)
+    assert "mfma_256" in name, name
+
+
+@pytest.mark.parametrize("shape", [(33, 4, 16), (100, 260, 48), (257, 1028, 64), (1000, 12, 512),
+                                   (1, 1, 8), (31, 33, 8), (100, 10, 64), (65, 37, 24),
+                                   (20000, 10, 512), (7, 1000, 40)])
+@pytest.mark.parametrize("pad_cols", [4, 1])
+def test_small_kernel_ragged_shapes(handle, torch_gpu, oracle, rng, shape, pad_cols):
+    """Any M and N, K a multiple of 8, go through the 32x32 k-split kernel; output rows need
+    no alignment (pad_cols = 1 gives an odd leading dimension)."""
+    name = ragged_check(handle, torch_gpu, oracle, rng, ci.ALGO_SMALL, shape, pad_cols)
+    assert "small" in name, name
+
+
+def test_default_choice_by_shape(handle, torch_gpu):
+    """Small problems and narrow outputs go to the 32x32 kernel, large ones to 256-column
+    tiles, what neither takes to the any-shape kernel."""
+    torch = torch_gpu
+    def kernel_for(M, N, K):
+        handle.gemm_f32(torch.zeros((M, K), device="cuda"), torch.zeros((K, N), device="cuda"))
+        return handle.last_kernel
+    assert handle.get_algo() == ci.ALGO_DEFAULT
+    assert "small" in kernel_for(512, 512, 512)
+    assert "small" in kernel_for(1024, 1024, 1024)
+    assert "small" in kernel_for(20000, 10, 512)
+    assert "mfma_256" in kernel_for(2048, 2048, 2048)
+    assert "mfma_256" in kernel_for(4096, 4096, 64)
+    assert "mfma_256" in kernel_for(20000, 512, 784)
+    assert "generic" in kernel_for(77, 91, 300)
+
+
+def test_all_kernels_agree_on_exact_inputs(handle, torch_gpu, oracle, rng):
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    A = rng.choice(vals, size=(300, 128))
+    B = rng.choice(vals, size=(128, 260))
+    want = oracle.gemm_f32(A, B)
+    for algo in (ci.ALGO_GENERIC, ci.ALGO_TILE, ci.ALGO_SMALL, ci.ALGO_DEFAULT):
+        with handle.algo(algo):
+            np.testing.assert_array_equal(run(handle, torch_gpu, A, B), want)

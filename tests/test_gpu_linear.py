@@ -8,12 +8,13 @@ import cudaintro_amd as ci
 pytestmark = pytest.mark.gpu
 
 
-def check(handle, torch, oracle, X, W, bias, relu, expect_mfma=None):
-    out = handle.linear_f32(torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda(),
-                            torch.from_numpy(bias).cuda() if bias is not None else None,
-                            ci.ACT_RELU if relu else ci.ACT_NONE).cpu().numpy()
-    if expect_mfma is not None:
-        assert ("mfma" in handle.last_kernel) == expect_mfma, handle.last_kernel
+def check(handle, torch, oracle, X, W, bias, relu, expect=None, algo=ci.ALGO_DEFAULT):
+    with handle.algo(algo):
+        out = handle.linear_f32(torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda(),
+                                torch.from_numpy(bias).cuda() if bias is not None else None,
+                                ci.ACT_RELU if relu else ci.ACT_NONE).cpu().numpy()
+    if expect is not None:
+        assert expect in handle.last_kernel, handle.last_kernel
     cpu = oracle.linear_f32(X, W, bias, relu)
     # fp32 gate of the GEMM path: |gpu - cpu| <= 1e-5 * max(|cpu|, rms of the pre-activation)
     pre = oracle.linear_f32(X, W, bias, False)
@@ -31,16 +32,16 @@ def test_mnist_hidden_layer(handle, torch_gpu, oracle, rng):
     X = rng.uniform(0, 1, size=(20000, 784)).astype(np.float32)
     W = (rng.normal(size=(784, 512)) * np.sqrt(2.0 / 784)).astype(np.float32)
     b = rng.normal(size=512).astype(np.float32) * 0.1
-    out = check(handle, torch_gpu, oracle, X, W, b, True, expect_mfma=True)
+    out = check(handle, torch_gpu, oracle, X, W, b, True, expect="mfma_256")
     assert (out == 0).mean() > 0.1      # ReLU actually clips something
 
 
 def test_mnist_output_layer(handle, torch_gpu, oracle, rng):
-    """20000 x 512 -> 10, no activation: N = 10 is served by the any-shape kernel."""
+    """20000 x 512 -> 10, no activation: N = 10 goes to the 32x32 k-split kernel."""
     X = np.maximum(rng.normal(size=(20000, 512)), 0).astype(np.float32)
     W = (rng.normal(size=(512, 10)) * 0.05).astype(np.float32)
     b = rng.normal(size=10).astype(np.float32) * 0.1
-    check(handle, torch_gpu, oracle, X, W, b, False, expect_mfma=False)
+    check(handle, torch_gpu, oracle, X, W, b, False, expect="small")
 
 
 @pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 7), (64, 64, 64), (100, 48, 260), (257, 16, 12), (512, 512, 512)])
@@ -52,6 +53,20 @@ def test_shapes(handle, torch_gpu, oracle, rng, shape, relu, with_bias):
     W = rng.uniform(-1, 1, size=(K, N)).astype(np.float32)
     b = rng.uniform(-1, 1, size=N).astype(np.float32) if with_bias else None
     check(handle, torch_gpu, oracle, X, W, b, relu)
+
+
+@pytest.mark.parametrize("algo,shape", [
+    (ci.ALGO_GENERIC, (100, 48, 260)), (ci.ALGO_TILE, (100, 48, 260)), (ci.ALGO_SMALL, (100, 48, 260)),
+    (ci.ALGO_SMALL, (257, 16, 10)), (ci.ALGO_SMALL, (40, 512, 33)), (ci.ALGO_TILE, (300, 64, 512))])
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_each_kernel_family(handle, torch_gpu, oracle, rng, algo, shape, relu, with_bias):
+    M, K, N = shape
+    X = rng.uniform(-1, 1, size=(M, K)).astype(np.float32)
+    W = rng.uniform(-1, 1, size=(K, N)).astype(np.float32)
+    b = rng.uniform(-1, 1, size=N).astype(np.float32) if with_bias else None
+    expect = {ci.ALGO_GENERIC: "generic", ci.ALGO_TILE: "mfma_256", ci.ALGO_SMALL: "small"}[algo]
+    check(handle, torch_gpu, oracle, X, W, b, relu, expect=expect, algo=algo)
 
 
 def test_exact_inputs_bit_exact(handle, torch_gpu, oracle, rng):
