@@ -68,6 +68,9 @@ SIGNATURES = {
     "cigemmGetLastErrorString": (C.c_char_p, [_vp]),
     "cigemmGetVersion": (_ci, []),
     "cigemmGetLastKernelName": (C.c_char_p, [_vp]),
+    "cigemm_matrixMulTiled": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
+    "cigemm_matrixMulMatrixCores": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
+    "cigemm_matrixMulMatrixCoresBfloat16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
     "cigemmSetAlgo": (C.c_int, [_vp, C.c_int]),
     "cigemmGetAlgo": (C.c_int, [_vp, C.POINTER(C.c_int)]),
     "cigemm_gemm_f32": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
@@ -221,6 +224,30 @@ class Handle:
         torch = _torch()
         assert A.dtype == torch.float16 and B.dtype == torch.float16
         return self._gemm("cigemm_gemm_f16", A, B, out, torch.float16)
+
+    # -- study kernels (TileProgramming demo) -------------------------------------------------
+    def matrixMulTiled(self, A, B):
+        torch = _torch()
+        w = A.shape[0]
+        assert A.dtype == torch.float32 and A.shape == (w, w) and B.shape == (w, w)
+        assert A.is_contiguous() and B.is_contiguous()
+        Cm = torch.empty((w, w), dtype=torch.float32, device=A.device)
+        st = self.lib.cigemm_matrixMulTiled(self._h, Cm.data_ptr(), A.data_ptr(), B.data_ptr(), w)
+        self._check(st, "cigemm_matrixMulTiled")
+        return Cm
+
+    def matrixMulMatrixCores(self, A, B):
+        """A, B fp16 or bf16 square tensors; fp32 result."""
+        torch = _torch()
+        w = A.shape[0]
+        assert A.dtype == B.dtype and A.dtype in (torch.float16, torch.bfloat16)
+        assert A.shape == (w, w) and B.shape == (w, w) and A.is_contiguous() and B.is_contiguous()
+        name = ("cigemm_matrixMulMatrixCores" if A.dtype == torch.float16
+                else "cigemm_matrixMulMatrixCoresBfloat16")
+        Cm = torch.empty((w, w), dtype=torch.float32, device=A.device)
+        st = getattr(self.lib, name)(self._h, A.data_ptr(), B.data_ptr(), Cm.data_ptr(), w)
+        self._check(st, name)
+        return Cm
 
     def gemm_bf16(self, A, B, out=None):
         torch = _torch()

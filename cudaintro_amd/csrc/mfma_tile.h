@@ -475,7 +475,9 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
       const u32x4 v = *reinterpret_cast<const u32x4*>(scr + rl * ROW_STRIDE + c16 * 16);
       // N * OB is a multiple of 16: a 16-byte piece is in or out as a whole
       if (row0 + rl < M && n0 + wn * 128 + c16 * (16 / OB) < N)
-        *reinterpret_cast<u32x4*>(epi.out_row(row0 + rl) + (n0 + wn * 128) * OB + c16 * 16) = v;
+        // streaming store: C is not read again by this kernel and should not evict A / B
+        __builtin_nontemporal_store(
+            v, reinterpret_cast<u32x4*>(epi.out_row(row0 + rl) + (n0 + wn * 128) * OB + c16 * 16));
     }
   }
 }

@@ -170,6 +170,27 @@ CIGEMM_API cigemmStatus_t cigemm_linear_f32(cigemmHandle_t handle, int64_t M, in
                                             const float* W, int64_t ldw, const float* bias,
                                             cigemmActivation_t act, float* out, int64_t ldo);
 
+/* ---- study kernels (TileProgramming demo) ---------------------------------------------- */
+
+/* C[width x width] = A . B, fp32, row-major, any width: the LDS-tiled 32x32 kernel.  Replaces
+ * matrixMulTiled<<<grid, block>>>(d_C, d_A, d_B, width) (TileProgramming/kernel.cu:54-102,
+ * launch 143-146) and launchMatrixMulCudaCores(C, A, B, width) (matmulTensor.cu:99-135).
+ * Products and sums are rounded separately in ascending k: the result equals matrixMulCPU
+ * (tensor_utils.cu:34-45) bit for bit. */
+CIGEMM_API cigemmStatus_t cigemm_matrixMulTiled(cigemmHandle_t handle, float* C, const float* A,
+                                                const float* B, int width);
+
+/* C[width x width] (fp32) = A . B with A, B fp16 / bf16 bit patterns, row-major, any width:
+ * one wavefront and one 32x32x16 matrix-core instruction per tile and 16 k.  Replace
+ * launchMatrixMulTensorCores(A, B, C, width) and launchMatrixMulTensorCoresBfloat16
+ * (TileProgramming/matmulTensor.cu:31-87), with both operands read row-major. */
+CIGEMM_API cigemmStatus_t cigemm_matrixMulMatrixCores(cigemmHandle_t handle, const uint16_t* A,
+                                                      const uint16_t* B, float* C, int width);
+CIGEMM_API cigemmStatus_t cigemm_matrixMulMatrixCoresBfloat16(cigemmHandle_t handle,
+                                                              const uint16_t* A,
+                                                              const uint16_t* B, float* C,
+                                                              int width);
+
 /* ---- device-side input generation -------------------------------------------------- */
 
 /* Replace fill_random_fp32 / _bf16 / _fp16 / _int8 (quantization/GEMM_fp32.cu:7-17,
