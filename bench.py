@@ -118,6 +118,7 @@ def main():
     handle = ci.Handle()
     n = args.size
     per_config = {}
+    mfma_probe = {}
 
     if args.copy_calibration:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")   # 1 GiB
@@ -263,8 +264,21 @@ def main():
                                                "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
                                                "bytes": nbytes, "kernel": handle.last_kernel}
             del wqs
+        # What the matrix cores sustain with no memory traffic at all, at the clock the chip
+        # holds under that load, on constant and on random operand bits.
+        probe = {}
+        for kind in ("bf16", "f16", "i8"):
+            for rnd in (False, True):
+                ops_box = [0]
+
+                def fnp():
+                    ops_box[0] = handle.probe_mfma(kind, rnd, 20000)
+                w, e = time_calls(torch, fnp, 3, 1)
+                probe[f"{kind}_{'random' if rnd else 'constant'}_bits"] = ops_box[0] * 3 / e / 1e12
+        mfma_probe.update(probe)
         for k, v in per_config.items():
             log(f"[bench]   {k}: {json.dumps(v)}")
+        log(f"[bench]   register-resident MFMA loop, T(FL)OP/s: {json.dumps(probe)}")
 
     line = {
         "metric": "GEMM TFLOPS/TOPS at 8192^3 per dtype (int8/bf16/fp16) + % of MFMA peak",
@@ -284,6 +298,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "per_config": per_config,
+        "mfma_only_probe": mfma_probe,
     }
     print(json.dumps(line), flush=True)
 

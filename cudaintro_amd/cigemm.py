@@ -71,6 +71,7 @@ SIGNATURES = {
     "cigemm_matrixMulTiled": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
     "cigemm_matrixMulMatrixCores": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
     "cigemm_matrixMulMatrixCoresBfloat16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
+    "cigemm_probe_mfma": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int64)]),
     "cigemmSetAlgo": (C.c_int, [_vp, C.c_int]),
     "cigemmGetAlgo": (C.c_int, [_vp, C.POINTER(C.c_int)]),
     "cigemm_gemm_f32": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
@@ -224,6 +225,14 @@ class Handle:
         torch = _torch()
         assert A.dtype == torch.float16 and B.dtype == torch.float16
         return self._gemm("cigemm_gemm_f16", A, B, out, torch.float16)
+
+    def probe_mfma(self, kind: str, random_bits: bool, iters: int) -> int:
+        """Launch the register-resident matrix-core loop; returns the operations it performs."""
+        ops = C.c_int64(0)
+        k = {"bf16": 0, "f16": 1, "i8": 2}[kind]
+        self._check(self.lib.cigemm_probe_mfma(self._h, k, int(random_bits), iters, C.byref(ops)),
+                    "cigemm_probe_mfma")
+        return ops.value
 
     # -- study kernels (TileProgramming demo) -------------------------------------------------
     def matrixMulTiled(self, A, B):

@@ -191,6 +191,17 @@ CIGEMM_API cigemmStatus_t cigemm_matrixMulMatrixCoresBfloat16(cigemmHandle_t han
                                                               const uint16_t* B, float* C,
                                                               int width);
 
+/* ---- measurement aid ------------------------------------------------------------------ */
+
+/* No counterpart in the reference.  Launches a register-resident matrix-core loop (no memory
+ * traffic inside the loop) on every compute unit of the handle's device, on the handle's
+ * stream: kind 0 = bf16 32x32x16, 1 = fp16 32x32x16, 2 = int8 32x32x32; random_bits 0 =
+ * constant operands, 1 = pseudo-random operand bits (sustained clocks depend on the data);
+ * `iters` loop trips of 16 instructions per wave.  *ops_per_launch receives 2.M.N.K summed
+ * over all instructions, for the caller to divide by the time it measures. */
+CIGEMM_API cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t handle, int kind, int random_bits,
+                                            int iters, int64_t* ops_per_launch);
+
 /* ---- device-side input generation -------------------------------------------------- */
 
 /* Replace fill_random_fp32 / _bf16 / _fp16 / _int8 (quantization/GEMM_fp32.cu:7-17,
