@@ -48,12 +48,19 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // ---- element conversions (device) -----------------------------------------------------
-// bfloat16: round to nearest even on the bit pattern; NaN keeps its sign and is quieted.
+// bfloat16: the gfx950 conversion instruction (v_cvt_pk_bf16_f32) rounds to nearest even and
+// quiets a NaN by setting mantissa bit 6 of the truncated pattern: on all 2^32 inputs it
+// returns what the bit-pattern rule "u += 0x7FFF + ((u >> 16) & 1); NaN -> (u >> 16) | 0x40"
+// returns.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16_bits(float lo, float hi) {
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
   return __builtin_bit_cast(float, (uint32_t)h << 16);
@@ -63,6 +70,10 @@ __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
   _Float16 h = (_Float16)f;
   return __builtin_bit_cast(uint16_t, h);
 }
+__device__ __forceinline__ uint32_t f32x2_to_f16_bits(float lo, float hi) {
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
   return (float)__builtin_bit_cast(_Float16, h);
 }
@@ -71,10 +82,16 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
 struct BF16 {
   static __device__ __forceinline__ float widen(uint16_t h) { return bf16_bits_to_f32(h); }
   static __device__ __forceinline__ uint16_t narrow(float f) { return f32_to_bf16_bits(f); }
+  static __device__ __forceinline__ uint32_t narrow2(float lo, float hi) {
+    return f32x2_to_bf16_bits(lo, hi);
+  }
 };
 struct F16 {
   static __device__ __forceinline__ float widen(uint16_t h) { return f16_bits_to_f32(h); }
   static __device__ __forceinline__ uint16_t narrow(float f) { return f32_to_f16_bits(f); }
+  static __device__ __forceinline__ uint32_t narrow2(float lo, float hi) {
+    return f32x2_to_f16_bits(lo, hi);
+  }
 };
 
 // ---- epilogues --------------------------------------------------------------------------

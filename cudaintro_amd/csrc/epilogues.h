@@ -23,8 +23,8 @@ struct EpiStore16x4 {
   __device__ __forceinline__ u32x2 pack(int64_t, int64_t, float v0, float v1, float v2,
                                         float v3) const {
     u32x2 v;
-    v[0] = (uint32_t)E16::narrow(v0) | ((uint32_t)E16::narrow(v1) << 16);
-    v[1] = (uint32_t)E16::narrow(v2) | ((uint32_t)E16::narrow(v3) << 16);
+    v[0] = E16::narrow2(v0, v1);
+    v[1] = E16::narrow2(v2, v3);
     return v;
   }
   __device__ __forceinline__ char* out_row(int64_t r) const {
@@ -139,8 +139,8 @@ struct EpiDequantX4 {
     o[3] = __fmul_rn(__fmul_rn((float)v3, a), b[3]);
     if constexpr (OUT_BF16) {
       u32x2 p;
-      p[0] = (uint32_t)f32_to_bf16_bits(o[0]) | ((uint32_t)f32_to_bf16_bits(o[1]) << 16);
-      p[1] = (uint32_t)f32_to_bf16_bits(o[2]) | ((uint32_t)f32_to_bf16_bits(o[3]) << 16);
+      p[0] = f32x2_to_bf16_bits(o[0], o[1]);
+      p[1] = f32x2_to_bf16_bits(o[2], o[3]);
       return p;
     } else {
       return __builtin_bit_cast(u32x4, f32x4{o[0], o[1], o[2], o[3]});
