@@ -1,7 +1,10 @@
 // Epilogue functors shared by the MFMA kernel families.  An epilogue turns four consecutive
 // accumulators of one output row (columns col..col+3) into output bits:
-//   pack(row, col, v0..v3)   the 4 output elements as raw bits (u32x2 for 16-bit outputs,
-//                            u32x4 for 32-bit ones); no memory is written;
+//   load_row(row)            what the epilogue needs per output row (a scale), fetched once;
+//   load_cols(col)           what it needs for the four columns col..col+3 (scales, bias);
+//   pack(rowv, colv, v0..v3) the 4 output elements as raw bits (u32x2 for 16-bit outputs,
+//                            u32x4 for 32-bit ones) from those; no memory is touched;
+//   pack(row, col, v0..v3)   the same with both fetched on the spot;
 //   side(row, col, v0..v3)   any second output of the same quad (the accumulator dump);
 //   out_row(row)             byte address of column 0 of that output row;
 //   operator()               pack + direct store (used where rows are not staged in LDS);
@@ -14,12 +17,22 @@
 
 namespace cig {
 
+struct EpiNothing {};
+
 // Narrows four consecutive columns and stores them as one 8-byte piece.
 template <typename E16>
 struct EpiStore16x4 {
   uint16_t* C;
   int64_t ldc;
   static constexpr int OUT_BYTES = 2;
+  typedef EpiNothing row_t;
+  typedef EpiNothing col_t;
+  __device__ __forceinline__ row_t load_row(int64_t) const { return row_t{}; }
+  __device__ __forceinline__ col_t load_cols(int64_t) const { return col_t{}; }
+  __device__ __forceinline__ u32x2 pack(row_t, col_t, float v0, float v1, float v2,
+                                        float v3) const {
+    return pack(0, 0, v0, v1, v2, v3);
+  }
   __device__ __forceinline__ u32x2 pack(int64_t, int64_t, float v0, float v1, float v2,
                                         float v3) const {
     u32x2 v;
@@ -42,6 +55,14 @@ struct EpiStoreF32x4 {
   float* C;
   int64_t ldc;
   static constexpr int OUT_BYTES = 4;
+  typedef EpiNothing row_t;
+  typedef EpiNothing col_t;
+  __device__ __forceinline__ row_t load_row(int64_t) const { return row_t{}; }
+  __device__ __forceinline__ col_t load_cols(int64_t) const { return col_t{}; }
+  __device__ __forceinline__ u32x4 pack(row_t, col_t, float v0, float v1, float v2,
+                                        float v3) const {
+    return pack(0, 0, v0, v1, v2, v3);
+  }
   __device__ __forceinline__ u32x4 pack(int64_t, int64_t, float v0, float v1, float v2,
                                         float v3) const {
     return __builtin_bit_cast(u32x4, f32x4{v0, v1, v2, v3});
@@ -64,11 +85,17 @@ struct EpiBiasActF32x4 {
   int64_t ldc;
   const float* bias;
   static constexpr int OUT_BYTES = 4;
-  __device__ __forceinline__ u32x4 pack(int64_t, int64_t c, float v0, float v1, float v2,
+  typedef EpiNothing row_t;
+  typedef f32x4 col_t;  // bias of the four columns
+  __device__ __forceinline__ row_t load_row(int64_t) const { return row_t{}; }
+  __device__ __forceinline__ col_t load_cols(int64_t c) const {
+    if (HAS_BIAS) return *reinterpret_cast<const f32x4*>(bias + c);
+    return f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  __device__ __forceinline__ u32x4 pack(row_t, col_t b, float v0, float v1, float v2,
                                         float v3) const {
     f32x4 v = {v0, v1, v2, v3};
     if (HAS_BIAS) {
-      const f32x4 b = *reinterpret_cast<const f32x4*>(bias + c);
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = __fadd_rn(v[e], b[e]);
     }
@@ -77,6 +104,10 @@ struct EpiBiasActF32x4 {
       for (int e = 0; e < 4; ++e) v[e] = fmaxf(0.0f, v[e]);
     }
     return __builtin_bit_cast(u32x4, v);
+  }
+  __device__ __forceinline__ u32x4 pack(int64_t r, int64_t c, float v0, float v1, float v2,
+                                        float v3) const {
+    return pack(load_row(r), load_cols(c), v0, v1, v2, v3);
   }
   __device__ __forceinline__ char* out_row(int64_t r) const {
     return reinterpret_cast<char*>(C + r * ldc);
@@ -95,6 +126,14 @@ struct EpiStoreI32x4 {
   int32_t* C;
   int64_t ldc;
   static constexpr int OUT_BYTES = 4;
+  typedef EpiNothing row_t;
+  typedef EpiNothing col_t;
+  __device__ __forceinline__ row_t load_row(int64_t) const { return row_t{}; }
+  __device__ __forceinline__ col_t load_cols(int64_t) const { return col_t{}; }
+  __device__ __forceinline__ u32x4 pack(row_t, col_t, int32_t v0, int32_t v1, int32_t v2,
+                                        int32_t v3) const {
+    return pack(0, 0, v0, v1, v2, v3);
+  }
   __device__ __forceinline__ u32x4 pack(int64_t, int64_t, int32_t v0, int32_t v1, int32_t v2,
                                         int32_t v3) const {
     return __builtin_bit_cast(u32x4, i32x4{v0, v1, v2, v3});
@@ -124,14 +163,16 @@ struct EpiDequantX4 {
   int64_t ldacc;
   static constexpr int OUT_BYTES = OUT_BF16 ? 2 : 4;
   typedef typename std::conditional<OUT_BF16, u32x2, u32x4>::type packed_t;
-  __device__ __forceinline__ packed_t pack(int64_t r, int64_t c, int32_t v0, int32_t v1,
-                                           int32_t v2, int32_t v3) const {
-    const float a = sa[sa_vec ? r : 0];
-    f32x4 b;
-    if (sb_vec)
-      b = *reinterpret_cast<const f32x4*>(sb + c);
-    else
-      b = f32x4{sb[0], sb[0], sb[0], sb[0]};
+  typedef float row_t;   // scale of the row
+  typedef f32x4 col_t;   // scales of the four columns
+  __device__ __forceinline__ row_t load_row(int64_t r) const { return sa[sa_vec ? r : 0]; }
+  __device__ __forceinline__ col_t load_cols(int64_t c) const {
+    if (sb_vec) return *reinterpret_cast<const f32x4*>(sb + c);
+    const float b0 = sb[0];
+    return f32x4{b0, b0, b0, b0};
+  }
+  __device__ __forceinline__ packed_t pack(row_t a, col_t b, int32_t v0, int32_t v1, int32_t v2,
+                                           int32_t v3) const {
     float o[4];
     o[0] = __fmul_rn(__fmul_rn((float)v0, a), b[0]);
     o[1] = __fmul_rn(__fmul_rn((float)v1, a), b[1]);
@@ -145,6 +186,10 @@ struct EpiDequantX4 {
     } else {
       return __builtin_bit_cast(u32x4, f32x4{o[0], o[1], o[2], o[3]});
     }
+  }
+  __device__ __forceinline__ packed_t pack(int64_t r, int64_t c, int32_t v0, int32_t v1,
+                                           int32_t v2, int32_t v3) const {
+    return pack(load_row(r), load_cols(c), v0, v1, v2, v3);
   }
   __device__ __forceinline__ char* out_row(int64_t r) const {
     return static_cast<char*>(out) + r * ldo * OUT_BYTES;

@@ -447,13 +447,25 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   constexpr int LANES_PER_ROW = ROW_BYTES / 16;
   constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
   char* scr = lds + w * (32 * ROW_STRIDE);
-  typedef decltype(epi.pack(0, 0, acc[0][0][0], acc[0][0][0], acc[0][0][0], acc[0][0][0])) packed_t;
+  typedef decltype(epi.pack((int64_t)0, (int64_t)0, acc[0][0][0], acc[0][0][0], acc[0][0][0],
+                            acc[0][0][0])) packed_t;
+  // What the epilogue needs per column quad (scales, bias) is the same for every row tile:
+  // fetched once, up front, so that no load latency sits between the accumulator reads.
+  typename Epi::col_t colv[4][4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int64_t col = n0 + wn * 128 + 32 * j + 8 * q + 4 * g;
+      colv[j][q] = epi.load_cols(col < N ? col : N - 4);
+    }
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     const int64_t row0 = m0 + wm * 32 * MT + 32 * i;
     const int64_t row = row0 + (l & 31);
     const bool row_ok = row < M;
     const int64_t row_c = row_ok ? row : M - 1;  // scale lookups stay in bounds
+    const typename Epi::row_t rowv = epi.load_row(row_c);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -462,7 +474,7 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
         const int64_t col = n0 + wn * 128 + c;
         const bool col_ok = col < N;  // N is a multiple of 4: a quad is in or out as a whole
         *reinterpret_cast<packed_t*>(scr + (l & 31) * ROW_STRIDE + c * OB) =
-            epi.pack(row_c, col_ok ? col : N - 4, acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
+            epi.pack(rowv, colv[j][q], acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
                      acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
         if (row_ok && col_ok)
           epi.side(row, col, acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
