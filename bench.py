@@ -54,6 +54,19 @@ def time_calls(torch, fn, steps, warmup):
     return wall, e0.elapsed_time(e1) * 1e-3
 
 
+def median_call_ms(torch, fn, steps):
+    """Median over `steps` individually HIP-event-timed calls (each call bracketed by its own
+    pair of events on the launch stream)."""
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+           for _ in range(steps)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return float(np.median([a.elapsed_time(b) for a, b in evs]))
+
+
 def dev16(torch, bits, kind):
     if kind == "bf16":
         return torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
@@ -146,6 +159,8 @@ def main():
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_16BIT_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_16BIT_TFLOPS, "traffic": None, "kernel": kernel,
                 "avg_kernel_ms": ev / args.steps * 1e3}
+    roofline["median_kernel_ms"] = median_call_ms(torch, lambda: handle.gemm_bf16(A, B, out=C),
+                                                  max(50, args.steps))
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file):
         roofline["traffic"] = json.load(open(traffic_file)).get(f"bf16_{n}")

@@ -7,7 +7,7 @@
 namespace cig {
 namespace {
 
-constexpr int PROBE_UNROLL = 16;  // independent accumulators per wave
+constexpr int PROBE_UNROLL = 12;  // independent accumulators per wave (no register spills)
 
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
   x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;

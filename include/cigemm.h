@@ -198,7 +198,7 @@ CIGEMM_API cigemmStatus_t cigemm_matrixMulMatrixCoresBfloat16(cigemmHandle_t han
  * stream: kind 0 = bf16 32x32x16, 1 = fp16 32x32x16, 2 = int8 32x32x32, 3 = bf16 16x16x32,
  * 4 = fp16 16x16x32, 5 = int8 16x16x64; random_bits 0 =
  * constant operands, 1 = pseudo-random operand bits (sustained clocks depend on the data);
- * `iters` loop trips of 16 instructions per wave.  *ops_per_launch receives 2.M.N.K summed
+ * `iters` loop trips of 12 instructions per wave.  *ops_per_launch receives 2.M.N.K summed
  * over all instructions, for the caller to divide by the time it measures. */
 CIGEMM_API cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t handle, int kind, int random_bits,
                                             int iters, int64_t* ops_per_launch);

@@ -108,7 +108,7 @@ def test_matrix_core_probe(handle, torch_gpu):
     import ctypes
     ops = handle.probe_mfma("bf16", True, 10)
     cus = torch_gpu.cuda.get_device_properties(0).multi_processor_count
-    assert ops == cus * 4 * 10 * 16 * 32768
+    assert ops == cus * 4 * 10 * 12 * 32768
     assert handle.probe_mfma("i8", False, 10) == 2 * ops
     assert handle.probe_mfma("bf16_16x16", False, 10) == ops // 2
     assert handle.probe_mfma("i8_16x16", False, 10) == ops
