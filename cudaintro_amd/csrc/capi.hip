@@ -90,7 +90,7 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->last_kernel = "";
   ctx->algo = CIGEMM_ALGO_DEFAULT;
   ctx->last_error[0] = '\0';
-  ctx->ws_partial_bytes = (size_t)16 << 20;
+  ctx->ws_partial_bytes = (size_t)64 << 20;
   ctx->ws_counter_bytes = (size_t)64 << 10;
   ctx->workspace = nullptr;
   if (hipMalloc(&ctx->workspace, ctx->ws_partial_bytes + ctx->ws_counter_bytes) != hipSuccess ||

@@ -13,13 +13,13 @@ bool launch_16b_mfma(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_
   if (!tile::tile_shape_ok(M, N, K, 2, A, lda, B, ldb, true) || N % 8) return false;
   if (ldc % 8 || ((uintptr_t)C & 15)) return false;  // output rows are stored in 16-byte pieces
   if (bf16) {
-    tile::launch_tile<tile::MathBF16, tile::B_KN16>(ctx, M, N, K * 2, A, lda * 2, B, ldb * 2,
-                                                    EpiStore16x4<BF16>{C, ldc});
-    ctx->last_kernel = "bf16_mfma_256x256x32_ring4";
+    const bool split = tile::launch_tile<tile::MathBF16, tile::B_KN16>(
+        ctx, M, N, K * 2, A, lda * 2, B, ldb * 2, EpiStore16x4<BF16>{C, ldc});
+    ctx->last_kernel = split ? "bf16_mfma_256x256x32_ring4_splitk" : "bf16_mfma_256x256x32_ring4";
   } else {
-    tile::launch_tile<tile::MathF16, tile::B_KN16>(ctx, M, N, K * 2, A, lda * 2, B, ldb * 2,
-                                                   EpiStore16x4<F16>{C, ldc});
-    ctx->last_kernel = "f16_mfma_256x256x32_ring4";
+    const bool split = tile::launch_tile<tile::MathF16, tile::B_KN16>(
+        ctx, M, N, K * 2, A, lda * 2, B, ldb * 2, EpiStore16x4<F16>{C, ldc});
+    ctx->last_kernel = split ? "f16_mfma_256x256x32_ring4_splitk" : "f16_mfma_256x256x32_ring4";
   }
   return true;
 }

@@ -40,21 +40,23 @@ bool launch_f32_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const 
                      const BiasAct* ba) {
   if (!f32_tile_ok(M, N, K, A, lda, B, ldb, C, ldc, ba)) return false;
   if (!ba) {
-    tile::launch_tile<tile::MathF32, tile::B_KN32>(ctx, M, N, K * 4, A, lda * 4, B, ldb * 4,
-                                                   EpiStoreF32x4{C, ldc});
-    ctx->last_kernel = "f32_mfma_256x256x16_ring4";
+    const bool split = tile::launch_tile<tile::MathF32, tile::B_KN32>(
+        ctx, M, N, K * 4, A, lda * 4, B, ldb * 4, EpiStoreF32x4{C, ldc});
+    ctx->last_kernel = split ? "f32_mfma_256x256x16_ring4_splitk" : "f32_mfma_256x256x16_ring4";
     return true;
   }
-#define CIG_BA(HB, RL)                                                                  \
-  tile::launch_tile<tile::MathF32, tile::B_KN32>(ctx, M, N, K * 4, A, lda * 4, B, ldb * 4, \
-                                                 EpiBiasActF32x4<HB, RL>{C, ldc, ba->bias})
+  bool split = false;
+#define CIG_BA(HB, RL)                                                                          \
+  split = tile::launch_tile<tile::MathF32, tile::B_KN32>(ctx, M, N, K * 4, A, lda * 4, B, ldb * 4, \
+                                                         EpiBiasActF32x4<HB, RL>{C, ldc, ba->bias})
   if (ba->bias) {
     if (ba->relu) CIG_BA(true, true); else CIG_BA(true, false);
   } else {
     if (ba->relu) CIG_BA(false, true); else CIG_BA(false, false);
   }
 #undef CIG_BA
-  ctx->last_kernel = "f32_mfma_256x256x16_ring4_bias_act";
+  ctx->last_kernel = split ? "f32_mfma_256x256x16_ring4_bias_act_splitk"
+                           : "f32_mfma_256x256x16_ring4_bias_act";
   return true;
 }
 

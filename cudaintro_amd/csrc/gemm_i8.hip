@@ -8,15 +8,15 @@ namespace cig {
 namespace {
 
 template <int BMODE>
-void launch_layout(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
+bool launch_layout(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
                    int64_t lda, const int8_t* B, int64_t ldb, int32_t* C, int64_t ldc,
                    const DequantArgs* dq) {
   if (!dq) {
-    tile::launch_tile<tile::MathI8, BMODE>(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32x4{C, ldc});
-    return;
+    return tile::launch_tile<tile::MathI8, BMODE>(ctx, M, N, K, A, lda, B, ldb,
+                                                  EpiStoreI32x4{C, ldc});
   }
 #define CIG_DQ(OB, DA)                                                                        \
-  tile::launch_tile<tile::MathI8, BMODE>(                                                     \
+  return tile::launch_tile<tile::MathI8, BMODE>(                                              \
       ctx, M, N, K, A, lda, B, ldb,                                                           \
       EpiDequantX4<OB, DA>{dq->out, dq->ldo, dq->sa, dq->sb, dq->sa_vec, dq->sb_vec,          \
                            dq->acc_out, dq->ldacc})
@@ -44,12 +44,14 @@ bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const i
     if (dq->sb_vec && ((uintptr_t)dq->sb & 15)) return false;
     if (dq->acc_out && (dq->ldacc % 4 || ((uintptr_t)dq->acc_out & 15))) return false;
   }
-  if (b_nk)
-    launch_layout<tile::B_NK>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
-  else
-    launch_layout<tile::B_KN8>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
-  ctx->last_kernel = dq ? (b_nk ? "i8_mfma_256x256x64_ring4_nk_dequant" : "i8_mfma_256x256x64_ring4_kn_dequant")
-                        : (b_nk ? "i8_mfma_256x256x64_ring4_nk" : "i8_mfma_256x256x64_ring4_kn");
+  const bool split = b_nk ? launch_layout<tile::B_NK>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq)
+                          : launch_layout<tile::B_KN8>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
+  static const char* const names[2][2][2] = {
+      {{"i8_mfma_256x256x64_ring4_kn", "i8_mfma_256x256x64_ring4_kn_splitk"},
+       {"i8_mfma_256x256x64_ring4_nk", "i8_mfma_256x256x64_ring4_nk_splitk"}},
+      {{"i8_mfma_256x256x64_ring4_kn_dequant", "i8_mfma_256x256x64_ring4_kn_dequant_splitk"},
+       {"i8_mfma_256x256x64_ring4_nk_dequant", "i8_mfma_256x256x64_ring4_nk_dequant_splitk"}}};
+  ctx->last_kernel = names[dq ? 1 : 0][b_nk ? 1 : 0][split ? 1 : 0];
   return true;
 }
 

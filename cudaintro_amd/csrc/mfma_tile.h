@@ -269,6 +269,41 @@ __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int&
   tn = in_group / gsize;
 }
 
+// Split-K: the accumulators of one K range, stored raw (fp32 or int32 bits) to
+// base + split * split_stride, row-major with leading dimension ld.
+struct EpiNone {};
+struct EpiPartialX4 {
+  uint32_t* base;
+  int64_t ld;
+  int64_t split_stride;  // elements between the partial matrices of consecutive splits
+  static constexpr int OUT_BYTES = 4;
+  typedef EpiNone row_t;
+  typedef EpiNone col_t;
+  __device__ __forceinline__ row_t load_row(int64_t) const { return row_t{}; }
+  __device__ __forceinline__ col_t load_cols(int64_t) const { return col_t{}; }
+  template <typename T>
+  __device__ __forceinline__ u32x4 pack(row_t, col_t, T v0, T v1, T v2, T v3) const {
+    return u32x4{__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1),
+                 __builtin_bit_cast(uint32_t, v2), __builtin_bit_cast(uint32_t, v3)};
+  }
+  template <typename T>
+  __device__ __forceinline__ u32x4 pack(int64_t, int64_t, T v0, T v1, T v2, T v3) const {
+    return pack(row_t{}, col_t{}, v0, v1, v2, v3);
+  }
+  __device__ __forceinline__ char* out_row(int64_t r) const {
+    return reinterpret_cast<char*>(base + r * ld);
+  }
+  template <typename T>
+  __device__ __forceinline__ void side(int64_t, int64_t, T, T, T, T) const {}
+  EpiPartialX4 shift_cols(int64_t c0) const { return EpiPartialX4{base + c0, ld, split_stride}; }
+};
+// The epilogue of K range `split` (blockIdx.y): only the partial store depends on it.
+template <typename Epi>
+__device__ __forceinline__ Epi epilogue_of_split(const Epi& e, int) { return e; }
+__device__ __forceinline__ EpiPartialX4 epilogue_of_split(const EpiPartialX4& e, int split) {
+  return EpiPartialX4{e.base + split * e.split_stride, e.ld, e.split_stride};
+}
+
 // Epi: __device__ void operator()(int64_t row, int64_t col, scalar v0, v1, v2, v3) stores the
 // four consecutive columns col..col+3 of one output row.
 //
@@ -281,7 +316,14 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
                                                            const char* __restrict__ A,
                                                            int64_t lda,
                                                            const char* __restrict__ B,
-                                                           int64_t ldb, Epi epi) {
+                                                           int64_t ldb, Epi epi_all,
+                                                           int64_t a_split_step,
+                                                           int64_t b_split_step) {
+  // blockIdx.y = K range (split-K launches only): KTS stages starting a_split_step /
+  // b_split_step bytes further per range
+  const Epi epi = epilogue_of_split(epi_all, (int)blockIdx.y);
+  A += blockIdx.y * a_split_step;
+  B += blockIdx.y * b_split_step;
   typedef typename Math::acc_t acc_t;
   typedef BTile<BMODE> BT;
   constexpr int DIST = NSTAGES - 1;  // stages in flight ahead of the one being multiplied
@@ -498,7 +540,8 @@ constexpr int DEFAULT_STAGES = 4;
 
 template <typename Math, int BMODE, int MT, typename Epi>
 void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
-                    int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi) {
+                    int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi,
+                    int splits = 1) {
   constexpr int NSTAGES = DEFAULT_STAGES;
   constexpr int LDS_BYTES = NSTAGES * STAGE_BYTES;
   auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, MT, Epi>;
@@ -509,10 +552,59 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
     attr_device = ctx->device;
   }
   const int tiles_m = (int)((M + 64 * MT - 1) / (64 * MT)), tiles_n = (int)((N + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), LDS_BYTES, ctx->stream,
-                     (int)M, (int)N, tiles_m, tiles_n, (int)(K_bytes / KB),
-                     static_cast<const char*>(A),
-                     lda_bytes, static_cast<const char*>(B), ldb_bytes, epi);
+  const int64_t kts = K_bytes / KB / splits;  // stages per K range
+  const int64_t a_step = kts * KB;
+  const int64_t b_step = BMODE == B_NK ? kts * KB : kts * (KB / Math::ELEM_BYTES) * ldb_bytes;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(256),
+                     LDS_BYTES, ctx->stream, (int)M, (int)N, tiles_m, tiles_n, (int)kts,
+                     static_cast<const char*>(A), lda_bytes, static_cast<const char*>(B),
+                     ldb_bytes, epi, a_step, b_step);
+}
+
+// Second half of a split-K GEMM: sums the `splits` partial matrices in split order (the
+// result does not depend on timing) and applies the real epilogue, four columns per lane.
+template <typename Scalar, typename Epi>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int splits,
+                                                            const uint32_t* __restrict__ part,
+                                                            int64_t split_stride, Epi epi) {
+  const int64_t quads_per_row = N / 4, quads = (int64_t)M * quads_per_row;
+  for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads;
+       q += (int64_t)gridDim.x * 256) {
+    const int64_t r = q / quads_per_row, c = (q % quads_per_row) * 4;
+    const uint32_t* p = part + r * N + c;
+    // (element-wise: a bit cast applied directly to a vector element misreads it)
+    auto as_scalar = [](uint32_t bits) { return __builtin_bit_cast(Scalar, bits); };
+    u32x4 v = *reinterpret_cast<const u32x4*>(p);
+    Scalar sum[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t b = v[e];
+      sum[e] = as_scalar(b);
+    }
+    for (int sp = 1; sp < splits; ++sp) {
+      v = *reinterpret_cast<const u32x4*>(p + sp * split_stride);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t b = v[e];
+        sum[e] += as_scalar(b);
+      }
+    }
+    epi(r, c, sum[0], sum[1], sum[2], sum[3]);
+  }
+}
+
+// Number of K ranges for a problem whose tiles would leave most of the chip idle: a power of
+// two that brings the workgroup count up to about the number of compute units, keeps at least
+// 8 stages per range, and whose partial matrices fit the handle's workspace.  1 = no split.
+inline int choose_tile_splits(const cigemmContext* ctx, int64_t M, int64_t N, int64_t kts,
+                              int64_t tiles) {
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  if (!ctx->workspace || tiles * 2 > cus) return 1;
+  int s = 1;
+  while (s < 16 && tiles * (2 * s) <= cus && kts % (2 * s) == 0 && kts / (2 * s) >= 8 &&
+         (size_t)(2 * s) * (size_t)M * (size_t)N * 4 <= ctx->ws_partial_bytes)
+    s *= 2;
+  return s;
 }
 
 // Relative cost of covering M x N with tiles of 64*mt rows on `cus` compute units: rounds of
@@ -539,25 +631,46 @@ inline int best_mt(int64_t M, int64_t N, int cus, double* cost = nullptr) {
 template <typename Math, int BMODE, typename Epi>
 void launch_tile_any_mt(cigemmContext* ctx, int mt, int64_t M, int64_t N, int64_t K_bytes,
                         const void* A, int64_t lda_bytes, const void* B, int64_t ldb_bytes,
-                        const Epi& epi) {
+                        const Epi& epi, int splits = 1) {
   if (mt == 4)
-    launch_tile_mt<Math, BMODE, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+    launch_tile_mt<Math, BMODE, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
   else if (mt == 2)
-    launch_tile_mt<Math, BMODE, 2>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+    launch_tile_mt<Math, BMODE, 2>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
   else
-    launch_tile_mt<Math, BMODE, 1>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+    launch_tile_mt<Math, BMODE, 1>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
 }
 
 // Chooses the tile height, and, when the last round of 256-row tiles would leave most of the
 // chip idle, covers the columns of the full rounds with 256-row tiles and the remaining
 // columns with a second launch of shorter tiles.  Epi::shift_cols(c) returns the epilogue of
 // the sub-problem starting at column c.
+// Returns true when the problem was run as a split-K pair of launches.
 template <typename Math, int BMODE, typename Epi>
-void launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
+bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
                  int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi) {
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
   double single = 0;
   const int mt = best_mt(M, N, cus, &single);
+  {
+    // Few tiles and a long K: split K over blockIdx.y, partial sums to the workspace, then
+    // one reduction launch with the real epilogue.
+    const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + BN - 1) / BN);
+    const int splits = choose_tile_splits(ctx, M, N, K_bytes / KB, tiles);
+    if (splits > 1) {
+      typedef typename Math::scalar_t scalar_t;
+      uint32_t* ws = static_cast<uint32_t*>(ctx->workspace);
+      const EpiPartialX4 part{ws, N, M * N};
+      launch_tile_any_mt<Math, BMODE>(ctx, mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, part,
+                                      splits);
+      const int64_t quads = M * (N / 4);
+      const unsigned grid = (unsigned)((quads + 255) / 256 < 4 * (int64_t)cus
+                                           ? (quads + 255) / 256
+                                           : 4 * (int64_t)cus);
+      hipLaunchKernelGGL((splitk_reduce_kernel<scalar_t, Epi>), dim3(grid), dim3(256), 0,
+                         ctx->stream, (int)M, (int)N, splits, ws, M * N, epi);
+      return true;
+    }
+  }
   {
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > cus && cus % tiles_m == 0) {
@@ -573,12 +686,13 @@ void launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
                            (BMODE == B_NK ? n1 * ldb_bytes : n1 * Math::ELEM_BYTES);
           launch_tile_any_mt<Math, BMODE>(ctx, mt2, M, n2, K_bytes, A, lda_bytes, B2, ldb_bytes,
                                           epi.shift_cols(n1));
-          return;
+          return false;
         }
       }
     }
   }
   launch_tile_any_mt<Math, BMODE>(ctx, mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+  return false;
 }
 
 // Shape / alignment gate shared by the families (sizes in elements, elem = bytes each;

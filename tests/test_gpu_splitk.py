@@ -1,0 +1,82 @@
+"""Split-K runs of the tile kernel (few output tiles, long K): partial sums per K range in the
+handle's workspace, then one reduction launch with the real epilogue."""
+import numpy as np
+import pytest
+
+import cudaintro_amd as ci
+from gpu_util import bits, error_bound_16, to_dev
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(33, 512, 2048), (64, 1024, 4096), (100, 260, 1024), (256, 2048, 8192), (300, 256, 1536)]
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_splitk_16bit(handle, torch_gpu, oracle, rng, kind, shape):
+    torch = torch_gpu
+    M, N, K = shape
+    if kind == "f16" and N % 8:
+        pytest.skip("16-bit output rows of the tile kernel are stored in 16-byte pieces")
+    narrow = oracle.f32_to_bf16 if kind == "bf16" else oracle.f32_to_f16
+    widen = oracle.bf16_to_f32 if kind == "bf16" else oracle.f16_to_f32
+    if N % 8:
+        pytest.skip("N must be a multiple of 8 for the 16-bit tile kernel")
+    Ab = narrow(rng.standard_normal((M, K)).astype(np.float32))
+    Bb = narrow(rng.standard_normal((K, N)).astype(np.float32))
+    fn = handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16
+    out = torch.full((M + 2, N + 8), 3.0, dtype=torch.bfloat16 if kind == "bf16" else torch.float16,
+                     device="cuda")
+    for _ in range(2):      # the workspace is reused: a second call must not see stale partials
+        fn(to_dev(torch, Ab, kind), to_dev(torch, Bb, kind), out=out[:M, :N])
+        assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+        ref, S = oracle.gemm_f64(widen(Ab), widen(Bb), with_abs=True)
+        o = widen(bits(torch, out))
+        assert (np.abs(o[:M, :N].astype(np.float64) - ref) <= error_bound_16(ref, S, K, kind)).all()
+        assert (o[M:] == 3.0).all() and (o[:, N:] == 3.0).all()
+
+
+@pytest.mark.parametrize("layout", [ci.B_KN, ci.B_NK])
+@pytest.mark.parametrize("shape", [(33, 512, 2048), (64, 1024, 4096), (100, 272, 1024), (256, 2048, 8192)])
+def test_splitk_int8(handle, torch_gpu, oracle, rng, layout, shape):
+    torch = torch_gpu
+    M, N, K = shape
+    A = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, size=(N, K) if layout == ci.B_NK else (K, N), dtype=np.int8)
+    acc_ref = oracle.gemm_i8_i32(A, B, b_is_nk=layout == ci.B_NK)
+    a, b = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    y = handle.gemm_i8_i32(a, b, layout)
+    assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+    np.testing.assert_array_equal(y.cpu().numpy(), acc_ref)
+    sa = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
+    sb = rng.uniform(1e-3, 5e-2, N).astype(np.float32)
+    for out_type, ot in (("f32", ci.OUT_F32), ("bf16", ci.OUT_BF16)):
+        out, acc = handle.gemm_i8_dequant(a, b, torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda(),
+                                          layout, ot, dump_acc=True)
+        assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+        np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
+        expect = oracle.dequant(acc_ref, sa, sb, out_dtype=out_type, sa_per_row=True, sb_per_col=True)
+        got = bits(torch, out) if out_type == "bf16" else out.cpu().numpy()
+        np.testing.assert_array_equal(got, expect)
+
+
+def test_splitk_f32_and_exact_inputs(handle, torch_gpu, oracle, rng):
+    torch = torch_gpu
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    M, N, K = 256, 512, 4096
+    A, B = rng.choice(vals, size=(M, K)), rng.choice(vals, size=(K, N))
+    bias = rng.choice(vals, size=N)
+    with handle.algo(ci.ALGO_TILE):
+        C = handle.gemm_f32(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()).cpu().numpy()
+        assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+        np.testing.assert_array_equal(C, oracle.gemm_f32(A, B))
+        L = handle.linear_f32(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(),
+                              torch.from_numpy(bias).cuda(), ci.ACT_RELU).cpu().numpy()
+        assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+        np.testing.assert_array_equal(L, oracle.linear_f32(A, B, bias, True))
+
+
+def test_large_shapes_do_not_split(handle, torch_gpu):
+    a = torch_gpu.zeros((2048, 2048), dtype=torch_gpu.bfloat16, device="cuda")
+    handle.gemm_bf16(a, a)
+    assert handle.last_kernel == "bf16_mfma_256x256x32_ring4"
