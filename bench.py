@@ -282,6 +282,27 @@ def main():
                                                "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
                                                "bytes": nbytes, "kernel": handle.last_kernel}
             del wqs
+        # small-batch shapes between the decode and the square configurations: few output
+        # tiles and a long K, run as split-K (weights still dominate the traffic)
+        for M in (64, 256):
+            xb, wb = wl.skinny_bf16(M, 8192, 8192, seed=4)
+            x = dev16(torch, xb, "bf16")
+            ws = [dev16(torch, wb, "bf16") for _ in range(4)]
+            y = torch.empty((M, 8192), dtype=torch.bfloat16, device="cuda")
+            it = [0]
+
+            def fnb():
+                handle.gemm_bf16(x, ws[it[0] & 3], out=y)
+                it[0] += 1
+            w, e = time_calls(torch, fnb, args.steps, args.warmup)
+            nbytes = wl.skinny_bytes(M, 8192, 8192, 2, 2, 2)
+            per_config[f"batch_bf16_M{M}"] = {"tflops": wl.gemm_ops(M, 8192, 8192) * args.steps / e / 1e12,
+                                              "gbs": nbytes * args.steps / e / 1e9,
+                                              "frac_of_peak": nbytes * args.steps / e / 1e9 / PEAK_HBM_GBS,
+                                              "peak": PEAK_HBM_GBS, "us": e / args.steps * 1e6,
+                                              "bytes": nbytes, "kernel": handle.last_kernel}
+            del ws
+
         # What the matrix cores sustain with no memory traffic at all, at the clock the chip
         # holds under that load, on constant and on random operand bits.
         probe = {}

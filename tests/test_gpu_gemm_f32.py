@@ -179,6 +179,8 @@ def test_default_choice_by_shape(handle, torch_gpu):
     assert "mfma_256" in kernel_for(2048, 2048, 2048)
     assert "mfma_256" in kernel_for(4096, 4096, 64)
     assert "mfma_256" in kernel_for(20000, 512, 784)
+    assert kernel_for(512, 512, 4096).endswith("_splitk")      # long K: tile kernel, K split
+    assert kernel_for(256, 1024, 8192).endswith("_splitk")
     assert "generic" in kernel_for(77, 91, 300)
 
 
