@@ -24,14 +24,16 @@ bool launch_f32_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const 
     // 157 us, small kernel 225 us; 1024^3: 74 us against 33 us; 512^3: 38 us against 8 us).
     const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
     double tile_cost = 0;
-    const int mt = tile::best_mt(M, N, cus, &tile_cost);
+    tile::best_mt(M, N, cus, &tile_cost);
     const double tiles32 = (double)((M + 31) / 32) * (double)((N + 31) / 32);
     const double small_cost = 0.115 * (tiles32 > cus ? tiles32 / cus : 1.0);
     // With a long K the tile kernel splits K over the idle compute units and wins
     // (512 x 512 x 4096: 33 us against 55 us; 1024^3: 31 against 32; 512^3: 17 against 9).
-    const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + tile::BN - 1) / tile::BN);
+    const bool one_round = ((M + 255) / 256) * ((N + tile::BN - 1) / tile::BN) <= cus;
     const bool long_k_split =
-        tile_ok && K >= 2048 && tile::choose_tile_splits(ctx, M, N, K * 4 / tile::KB, tiles) > 1;
+        tile_ok && K >= 2048 && one_round &&
+        tile::plan_small(ctx, M, N, K * 4 / tile::KB, tile::MathF32::STAGE_UNIT_US, K * 4 * N)
+                .splits > 1;
     if (!tile_ok || (small_cost < tile_cost && !long_k_split)) {
       launch_f32_small(ctx, M, N, K, A, lda, B, ldb, C, ldc, ba);
       return true;

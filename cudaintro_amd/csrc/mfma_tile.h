@@ -196,6 +196,7 @@ __device__ __forceinline__ typename BTile<MODE>::piece_t read_b_piece(const char
 // ---- arithmetic traits ----------------------------------------------------------------------
 struct MathBF16 {
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
+  static constexpr double STAGE_UNIT_US = 0.195;  // one 64 x 256 step of one 64-byte stage
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
   typedef f32x16 acc_t;
   typedef float scalar_t;
@@ -208,6 +209,7 @@ struct MathBF16 {
 };
 struct MathF16 {
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
+  static constexpr double STAGE_UNIT_US = 0.195;
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
   typedef f32x16 acc_t;
   typedef float scalar_t;
@@ -219,6 +221,7 @@ struct MathF16 {
 };
 struct MathI8 {
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
+  static constexpr double STAGE_UNIT_US = 0.195;
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
   typedef i32x16 acc_t;
   typedef int32_t scalar_t;
@@ -234,6 +237,7 @@ struct MathI8 {
 // so four MFMAs consume one fragment pair: MFMA e multiplies k0+e (lanes 0-31) and k0+4+e.
 struct MathF32 {
   static constexpr int SUBSTEPS = 4;
+  static constexpr double STAGE_UNIT_US = 0.95;
   static __device__ __forceinline__ float afrag(u32x4 a, int sub) {
     const uint32_t bits = a[sub];  // (bit_cast applied directly to a vector element misreads it)
     return __builtin_bit_cast(float, bits);
@@ -593,18 +597,43 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
   }
 }
 
-// Number of K ranges for a problem whose tiles would leave most of the chip idle: a power of
-// two that brings the workgroup count up to about the number of compute units, keeps at least
-// 8 stages per range, and whose partial matrices fit the handle's workspace.  1 = no split.
-inline int choose_tile_splits(const cigemmContext* ctx, int64_t M, int64_t N, int64_t kts,
-                              int64_t tiles) {
+// Plan for a problem that fits one round of 256-row tiles: tile height and number of K
+// ranges, by estimated time.  Main launch: rounds x tile cost x stages per range, where short
+// tiles cost more per output than in the compute-bound plan below because such problems are
+// bound by the weight stream (bf16 512 x 8192 x 8192, 256 workgroups each: 256-row tiles and
+// 4 ranges 85 us, 128-row and 2 ranges 89 us, 64-row unsplit 102 us).  Split plans add the
+// reduction launch: a fixed 5 us plus (splits + 1) M N 4 bytes at 3 TB/s.  `sm_us` = time of
+// one 64 x 256 x (64-byte stage) step of the arithmetic type; `b_bytes` = size of B: when it
+// stays in the caches the compute-bound tile costs apply.
+struct SmallPlan {
+  int mt;
+  int splits;
+};
+inline SmallPlan plan_small(const cigemmContext* ctx, int64_t M, int64_t N, int64_t kts,
+                            double sm_us, int64_t b_bytes) {
+  const bool streamed = b_bytes > (16LL << 20);
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-  if (!ctx->workspace || tiles * 2 > cus) return 1;
-  int s = 1;
-  while (s < 16 && tiles * (2 * s) <= cus && kts % (2 * s) == 0 && kts / (2 * s) >= 8 &&
-         (size_t)(2 * s) * (size_t)M * (size_t)N * 4 <= ctx->ws_partial_bytes)
-    s *= 2;
-  return s;
+  SmallPlan best{0, 1};
+  double best_us = 1e30;
+  for (int mt : {4, 2, 1}) {
+    if (mt > 1 && 64 * (mt / 2) >= M) continue;  // half the height already covers M
+    const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + BN - 1) / BN);
+    const double per_tile = mt == 4 ? 4.0 : mt == 2 ? (streamed ? 2.5 : 2.24) : (streamed ? 1.7 : 1.3);
+    for (int sp = 1; sp <= 16; sp *= 2) {
+      if (sp > 1) {
+        if (!ctx->workspace || kts % sp || kts / sp < 8) break;
+        if ((size_t)sp * (size_t)M * (size_t)N * 4 > ctx->ws_partial_bytes) break;
+      }
+      const double rounds = (double)((tiles * sp + cus - 1) / cus);
+      double us = rounds * per_tile * sm_us * (double)(kts / sp);
+      if (sp > 1) us += 5.0 + (double)(sp + 1) * (double)M * (double)N * 4.0 / 3.0e6;
+      if (us < best_us) {
+        best_us = us;
+        best = SmallPlan{mt, sp};
+      }
+    }
+  }
+  return best;
 }
 
 // Relative cost of covering M x N with tiles of 64*mt rows on `cus` compute units: rounds of
@@ -651,25 +680,27 @@ bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
   double single = 0;
   const int mt = best_mt(M, N, cus, &single);
-  {
-    // Few tiles and a long K: split K over blockIdx.y, partial sums to the workspace, then
-    // one reduction launch with the real epilogue.
-    const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + BN - 1) / BN);
-    const int splits = choose_tile_splits(ctx, M, N, K_bytes / KB, tiles);
-    if (splits > 1) {
+  if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) <= cus) {
+    // At most one round of 256-row tiles: pick the tile height and the number of K ranges
+    // together.  Split plans run K over blockIdx.y, partial sums to the workspace, then one
+    // reduction launch with the real epilogue.
+    const SmallPlan plan = plan_small(ctx, M, N, K_bytes / KB, Math::STAGE_UNIT_US, K_bytes * N);
+    if (plan.splits > 1) {
       typedef typename Math::scalar_t scalar_t;
       uint32_t* ws = static_cast<uint32_t*>(ctx->workspace);
       const EpiPartialX4 part{ws, N, M * N};
-      launch_tile_any_mt<Math, BMODE>(ctx, mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, part,
-                                      splits);
+      launch_tile_any_mt<Math, BMODE>(ctx, plan.mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes,
+                                      part, plan.splits);
       const int64_t quads = M * (N / 4);
       const unsigned grid = (unsigned)((quads + 255) / 256 < 4 * (int64_t)cus
                                            ? (quads + 255) / 256
                                            : 4 * (int64_t)cus);
       hipLaunchKernelGGL((splitk_reduce_kernel<scalar_t, Epi>), dim3(grid), dim3(256), 0,
-                         ctx->stream, (int)M, (int)N, splits, ws, M * N, epi);
+                         ctx->stream, (int)M, (int)N, plan.splits, ws, M * N, epi);
       return true;
     }
+    launch_tile_any_mt<Math, BMODE>(ctx, plan.mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+    return false;
   }
   {
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;

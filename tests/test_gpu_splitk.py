@@ -29,7 +29,9 @@ def test_splitk_16bit(handle, torch_gpu, oracle, rng, kind, shape):
                      device="cuda")
     for _ in range(2):      # the workspace is reused: a second call must not see stale partials
         fn(to_dev(torch, Ab, kind), to_dev(torch, Bb, kind), out=out[:M, :N])
-        assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+        if K >= 2048:
+            assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+        assert "mfma_256" in handle.last_kernel
         ref, S = oracle.gemm_f64(widen(Ab), widen(Bb), with_abs=True)
         o = widen(bits(torch, out))
         assert (np.abs(o[:M, :N].astype(np.float64) - ref) <= error_bound_16(ref, S, K, kind)).all()
@@ -46,14 +48,17 @@ def test_splitk_int8(handle, torch_gpu, oracle, rng, layout, shape):
     acc_ref = oracle.gemm_i8_i32(A, B, b_is_nk=layout == ci.B_NK)
     a, b = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
     y = handle.gemm_i8_i32(a, b, layout)
-    assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+    if K >= 2048:      # short K: the plan may well keep one K range
+        assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+    assert "mfma_256" in handle.last_kernel
     np.testing.assert_array_equal(y.cpu().numpy(), acc_ref)
     sa = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
     sb = rng.uniform(1e-3, 5e-2, N).astype(np.float32)
     for out_type, ot in (("f32", ci.OUT_F32), ("bf16", ci.OUT_BF16)):
         out, acc = handle.gemm_i8_dequant(a, b, torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda(),
                                           layout, ot, dump_acc=True)
-        assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+        if K >= 2048:
+            assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
         np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
         expect = oracle.dequant(acc_ref, sa, sb, out_dtype=out_type, sa_per_row=True, sb_per_col=True)
         got = bits(torch, out) if out_type == "bf16" else out.cpu().numpy()
