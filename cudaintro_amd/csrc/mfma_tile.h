@@ -5,9 +5,11 @@
 // owns a 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulators per lane (the AGPR
 // file); one wave per SIMD.  The tile height is a template parameter (MT = 4, 2 or 1 row
 // tiles per wave: 256, 128 or 64 rows) so that small or awkward M still fill the chip; the
-// text below describes MT = 4.  Both operand tiles of a stage are 16 KiB; NSTAGES (4 or 5) stages form
-// a ring in LDS (128 or 160 KiB), NSTAGES-1 of them in flight ahead of the one being
-// multiplied: HBM/L2 latency here is of the order of a microsecond, two to three stage times.
+// text below describes MT = 4.  Both operand tiles of a stage are 16 KiB.  B stages form a
+// ring of 4 slots in LDS (64 KiB), three of them in flight ahead of the one being multiplied:
+// HBM/L2 latency here is of the order of a microsecond, two to three stage times.  A is
+// fetched two stages at a time as whole 128-byte lines (half as many L2 requests as 64-byte
+// pieces) into a ring of 3 pair slots (96 KiB): 160 KiB in all.
 //
 // Global -> LDS goes straight through the LDS-DMA path (global_load_lds_dwordx4): no
 // staging registers, no ds_write.  One such instruction deposits the wave's 64 x 16 bytes
@@ -15,11 +17,12 @@
 // bank-conflict swizzle is therefore applied on the global side (the chunk a lane fetches),
 // and LDS slot s of a row holds chunk s ^ swizzle(row).
 //
-// A tile  [256 m][64 B of k], as in memory.  16-byte chunk c of row r lives at
-//         r*64 + ((c ^ fA(r)) << 4): the 16-byte fragment reads of 32 consecutive rows
-//         then spread over all banks.
+// A pair  [256 m][128 B of k] = stages 2p and 2p+1, as in memory.  16-byte chunk c of row r
+//         lives at r*128 + ((c ^ ((r >> 1) & 7)) << 4): the 16-byte fragment reads of 32
+//         consecutive rows then spread over all banks.
 // B tile  one of
-//   NK    [256 n][64 B of k]  (weights, k contiguous): same geometry and reads as A;
+//   NK    [256 n][64 B of k]  (weights, k contiguous): 16-byte chunk c of row r at
+//         r*64 + ((c ^ f(r)) << 4), read like A;
 //   KN16  [32 k][256 n] halves, KN8 [64 k][256 n] bytes (n contiguous, as C = A.B stores
 //         B).  The MFMA wants k contiguous per lane, so fragments come from the transposing
 //         LDS reads ds_read_b64_tr_b16 / _tr_b8: within 16 lanes, lane i supplies the
@@ -27,12 +30,13 @@
 //         k-values of column n0 + i.  Chunks are XOR-swizzled by k so that the rows one
 //         instruction touches fall in different banks.
 //
-// Pipeline, iteration s (stage s sits in ring slot s % NSTAGES):
+// Pipeline, iteration s (B of stage s sits in slot s % 4, A in pair slot (s / 2) % 3):
 //   k-step 0: 16 MFMAs on the fragments of (s,0); under them the 12 LDS reads of (s,1)
 //   wait until this wave's DMA of stage s+1 has landed (vmcnt), workgroup barrier
-//   k-step 1: 16 MFMAs on (s,1); under them the 12 LDS reads of (s+1,0) and the 8 DMA
-//             instructions of stage s+NSTAGES-1, into the slot stage s-1 just left (every
-//             wave finished reading it before it reached the barrier).
+//   k-step 1: 16 MFMAs on (s,1); under them the 12 LDS reads of (s+1,0) and the DMA of
+//             stage s+3: 4 instructions of B into the slot stage s-1 just left (every wave
+//             finished reading it before it reached the barrier) and, for odd s, the 8 of
+//             the A pair of stages s+3 and s+4.
 // Fragments are double buffered in registers.  The emitted order is pinned slot by slot
 // with scheduling fences: one MFMA, at most one LDS read, at most one DMA.
 //
@@ -66,6 +70,21 @@ __device__ __forceinline__ int rowmajor_swz(int r) {
 __device__ __forceinline__ int rowmajor_off(int r, int c) {
   return r * KB + ((c ^ rowmajor_swz(r)) << 4);
 }
+
+// ---- A pair tile: [64 T rows][128 B = two stages of k]: A is fetched as whole 128-byte lines,
+// one pair of stages at a time (half as many L2 requests as 64-byte pieces).  Chunk c (16 B)
+// of row r sits at r*128 + ((c ^ pair_swz(r)) << 4).
+__device__ __forceinline__ int pair_swz(int r) { return (r >> 1) & 7; }
+__device__ __forceinline__ int pair_off(int r, int c) { return r * 128 + ((c ^ pair_swz(r)) << 4); }
+// one instruction = 8 rows of 128 B; wave w moves rows 16 T w .. 16 T (w + 1): 2 T instructions
+template <int T>
+struct RowPairDmaT {
+  static __device__ __forceinline__ int dma_lds(int w, int i) { return (16 * T * w + 8 * i) * 128; }
+  static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld, int last) {
+    const int r = 16 * T * w + 8 * i + (l >> 3);
+    return (int64_t)(r < last ? r : last) * ld + (((l & 7) ^ pair_swz(r)) << 4);
+  }
+};
 
 enum BMode { B_NK = 0, B_KN16 = 1, B_KN8 = 2, B_KN32 = 3 };
 
@@ -332,8 +351,12 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   typedef BTile<BMODE> BT;
   constexpr int DIST = NSTAGES - 1;  // stages in flight ahead of the one being multiplied
   constexpr int TILE_M = 64 * MT;    // rows of the macro tile
-  constexpr int DMA_PER_STAGE = MT + 4;  // per wave: MT A + 4 B instructions of 1 KiB
-  typedef RowMajorDmaT<MT> ADma;
+  static_assert(NSTAGES == 4, "the wait counts below assume three stages in flight");
+  constexpr int DMA_A = 2 * MT;          // per wave and stage pair: A instructions of 1 KiB
+  constexpr int DMA_B = 4;               // per wave and stage: B instructions
+  constexpr int APAIR_BYTES = TILE_M * 128;
+  constexpr int B_RING = NSTAGES * OPERAND_BYTES;   // B slots first, then three A pair slots
+  typedef RowPairDmaT<MT> ADma;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int t = threadIdx.x;
   const int l = t & 63;
@@ -361,9 +384,21 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   const int a_last = (int)((M - 1 - m0) < (TILE_M - 1) ? (M - 1 - m0) : (TILE_M - 1));
   const int n_left = (int)((N - n0) < BN ? (N - n0) : BN);
   const int b_last = BMODE == B_NK ? n_left - 1 : n_left * Math::ELEM_BYTES / 16 - 1;
-  uint32_t a_voff[MT], b_voff[4];
+  // With an odd number of stages the last pair's second half lies past this K range (past
+  // the end of A for the last rows of the matrix): lanes that would fetch it fetch the first
+  // half again instead (bit i of a_hi = instruction i of this lane fetches chunk 4..7); that
+  // half of the slot is never read.
+  uint32_t a_hi = 0;
 #pragma unroll
-  for (int i = 0; i < MT; ++i) a_voff[i] = (uint32_t)ADma::dma_src(w, i, l, lda, a_last);
+  for (int i = 0; i < DMA_A; ++i) {
+    const int r = 16 * MT * w + 8 * i + (l >> 3);
+    a_hi |= (uint32_t)((((l & 7) ^ pair_swz(r)) >> 2) & 1) << i;
+  }
+  const int last_pair = (KTS - 1) >> 1;
+  const bool odd_kts = KTS & 1;
+  uint32_t a_voff[DMA_A], b_voff[4];
+#pragma unroll
+  for (int i = 0; i < DMA_A; ++i) a_voff[i] = (uint32_t)ADma::dma_src(w, i, l, lda, a_last);
 #pragma unroll
   for (int i = 0; i < 4; ++i) b_voff[i] = (uint32_t)BT::dma_src(w, i, l, ldb, b_last);
 
@@ -379,16 +414,21 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
                  : "s"(lds_dst), "v"(src)
                  : "m0");
   };
-  // DMA instruction d of stage `st` into ring slot `slot`: first the 4 of B, then the MT of A.
-  // Past the last stage the last one is fetched again (into a slot nobody reads any more),
-  // which keeps the number of outstanding instructions, and so the vmcnt waits, uniform.
-  auto dma_piece = [&](int st, int slot, int d) {
+  // d < 4: B instruction d of stage `st` into B slot `slot`; d >= 4: A instruction d - 4 of
+  // the stage pair st / 2 into pair slot `pslot`.  Past the last stage the last one is fetched
+  // again (into slots nobody reads any more), which keeps the number of outstanding
+  // instructions, and so the vmcnt waits, uniform.
+  auto dma_piece = [&](int st, int slot, int pslot, int d) {
     st = st < KTS ? st : KTS - 1;
-    const uint32_t sa = lds_base + slot * STAGE_BYTES;
     if (d < 4)
-      dma16(b_tile + (int64_t)st * b_kstep + b_voff[d], sa + OPERAND_BYTES + BT::dma_lds(w, d));
-    else
-      dma16(a_tile + (int64_t)st * KB + a_voff[d - 4], sa + ADma::dma_lds(w, d - 4));
+      dma16(b_tile + (int64_t)st * b_kstep + b_voff[d],
+            lds_base + slot * OPERAND_BYTES + BT::dma_lds(w, d));
+    else {
+      uint32_t off = a_voff[d - 4];
+      if (odd_kts && (st >> 1) == last_pair) off -= ((a_hi >> (d - 4)) & 1u) << 6;
+      dma16(a_tile + (int64_t)(st >> 1) * 128 + off,
+            lds_base + B_RING + pslot * APAIR_BYTES + ADma::dma_lds(w, d - 4));
+    }
   };
 
   const int a_frag_row = wm * 32 * MT + (l & 31);
@@ -398,18 +438,19 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   constexpr int NREAD = MT + BT::NREADS;               // LDS reads per k-step
   constexpr int NMFMA = 4 * MT * Math::SUBSTEPS;       // MFMAs per k-step
   constexpr int READS_PER_SLOT = (NREAD + NMFMA - 1) / NMFMA;
-  constexpr int DMA_PER_SLOT = (DMA_PER_STAGE + NMFMA - 1) / NMFMA;
+  constexpr int DMA_PER_SLOT = (DMA_B + DMA_A + NMFMA - 1) / NMFMA;
   struct Frags {
     u32x4 a[MT];
     typename BT::piece_t b[BT::NREADS];
   };
   // LDS read r of k-step kk of the stage in ring slot `slot`: first the A fragments, then B.
-  auto read_piece = [&](Frags& f, int slot, int kk, int r) {
-    const char* sa = lds + slot * STAGE_BYTES;
+  // `par` = parity of the stage: which half of the pair's 128-byte rows.
+  auto read_piece = [&](Frags& f, int slot, int pslot, int par, int kk, int r) {
     if (r < MT)
-      f.a[r] = *reinterpret_cast<const u32x4*>(sa + rowmajor_off(a_frag_row + 32 * r, 2 * kk + g));
+      f.a[r] = *reinterpret_cast<const u32x4*>(
+          lds + B_RING + pslot * APAIR_BYTES + pair_off(a_frag_row + 32 * r, 4 * par + 2 * kk + g));
     else
-      f.b[r - MT] = read_b_piece<BMODE>(sa + OPERAND_BYTES, wn, r - MT, kk, l);
+      f.b[r - MT] = read_b_piece<BMODE>(lds + slot * OPERAND_BYTES, wn, r - MT, kk, l);
   };
 
   acc_t acc[MT][4];
@@ -435,50 +476,67 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
     __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
   };
 
-  // prologue: stages 0 .. DIST-1 in flight; stage 0 landed; first fragments in registers
+  // prologue, in the order the main loop keeps: B[0], A pair 0, B[1], B[2], A pair 1; stage
+  // 0 landed; first fragments in registers
 #pragma unroll
-  for (int st = 0; st < DIST; ++st)
+  for (int d = 0; d < DMA_B + DMA_A; ++d) dma_piece(0, 0, 0, d);
 #pragma unroll
-    for (int d = 0; d < DMA_PER_STAGE; ++d) dma_piece(st, st, d);
-  wait_vmcnt(std::integral_constant<int, DMA_PER_STAGE*(DIST - 1)>{});
+  for (int d = 0; d < DMA_B; ++d) dma_piece(1, 1, 0, d);
+#pragma unroll
+  for (int d = 0; d < DMA_B + DMA_A; ++d) dma_piece(2, 2, 1, d);
+  wait_vmcnt(std::integral_constant<int, 2 * DMA_B + DMA_A>{});
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int r = 0; r < NREAD; ++r) read_piece(f0, 0, 0, r);
-
-  // Ring slots of the stage being multiplied, of the next one, and of the one the DMA fills
-  // (wave-uniform scalars, advanced modulo NSTAGES each iteration).
+  for (int r = 0; r < NREAD; ++r) read_piece(f0, 0, 0, 0, 0, r);
+  // B ring slots of the stage being multiplied, of the next one, and of the one the DMA
+  // fills (wave-uniform scalars, advanced modulo NSTAGES each stage); the three A pair slots
+  // likewise, advanced every second stage.
   int slot = 0, next_slot = 1, dma_slot = DIST;
-  for (int s = 0; s < KTS; ++s) {
-    // k-step 0
+  int pslot = 0, next_pslot = 1, dma_pslot = 2;
+  // One stage; PAR = its parity.  Even stages issue B[s+3] only; odd stages B[s+3] and the A
+  // pair of stages s+3, s+4.
+  auto stage = [&](int s, auto par_const) {
+    constexpr int PAR = decltype(par_const)::value;
+    constexpr int NDMA = PAR ? DMA_B + DMA_A : DMA_B;
 #pragma unroll
     for (int sl = 0; sl < NMFMA; ++sl) {
       mfma_piece(f0, sl);
 #pragma unroll
       for (int r = sl * READS_PER_SLOT; r < (sl + 1) * READS_PER_SLOT; ++r)
-        if (r < NREAD) read_piece(f1, slot, 1, r);
+        if (r < NREAD) read_piece(f1, slot, pslot, PAR, 1, r);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // stage s+1 landed for this wave (stages s+2 .. s+DIST-1 may still be in flight)
-    wait_vmcnt(std::integral_constant<int, DMA_PER_STAGE*(DIST - 2)>{});
+    // stage s+1 landed for this wave.  Still in flight, in issue order after what stage s+1
+    // needs: even s: B[s+2] and the A pair (s+2, s+3); odd s: B[s+2].
+    wait_vmcnt(std::integral_constant<int, PAR ? DMA_B : DMA_B + DMA_A>{});
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    // k-step 1
 #pragma unroll
     for (int sl = 0; sl < NMFMA; ++sl) {
       mfma_piece(f1, sl);
 #pragma unroll
       for (int r = sl * READS_PER_SLOT; r < (sl + 1) * READS_PER_SLOT; ++r)
-        if (r < NREAD) read_piece(f0, next_slot, 0, r);
+        if (r < NREAD) read_piece(f0, next_slot, PAR ? next_pslot : pslot, PAR ^ 1, 0, r);
 #pragma unroll
       for (int d = sl * DMA_PER_SLOT; d < (sl + 1) * DMA_PER_SLOT; ++d)
-        if (d < DMA_PER_STAGE) dma_piece(s + DIST, dma_slot, d);
+        if (d < NDMA) dma_piece(s + DIST, dma_slot, dma_pslot, d);
       __builtin_amdgcn_sched_barrier(0);
     }
     slot = next_slot;
     next_slot = next_slot + 1 == NSTAGES ? 0 : next_slot + 1;
     dma_slot = dma_slot + 1 == NSTAGES ? 0 : dma_slot + 1;
+    if (PAR) {
+      pslot = next_pslot;
+      next_pslot = next_pslot + 1 == 3 ? 0 : next_pslot + 1;
+      dma_pslot = dma_pslot + 1 == 3 ? 0 : dma_pslot + 1;
+    }
+  };
+  for (int s = 0; s + 1 < KTS; s += 2) {
+    stage(s, std::integral_constant<int, 0>{});
+    stage(s + 1, std::integral_constant<int, 1>{});
   }
+  if (KTS & 1) stage(KTS - 1, std::integral_constant<int, 0>{});  // odd stage count: the last one
   wait_vmcnt(std::integral_constant<int, 0>{});  // no DMA outlives the main loop
   __syncthreads();  // ... for any wave, and every wave is done reading the ring
 
@@ -547,7 +605,7 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
                     int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi,
                     int splits = 1) {
   constexpr int NSTAGES = DEFAULT_STAGES;
-  constexpr int LDS_BYTES = NSTAGES * STAGE_BYTES;
+  constexpr int LDS_BYTES = NSTAGES * OPERAND_BYTES + 3 * (64 * MT * 128);
   auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, MT, Epi>;
   static int attr_device = -1;  // one per template instance
   if (attr_device != ctx->device) {

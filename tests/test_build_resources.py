@@ -1,0 +1,49 @@
+"""Compile-only check of the register allocation of the hot kernels: a tile kernel that spills
+VGPRs to scratch runs several times slower and no numerics test notices.  Needs hipcc, no GPU."""
+import concurrent.futures
+import os
+import re
+import shutil
+import subprocess
+import tempfile
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "cudaintro_amd", "csrc")
+HIPCC = "/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else shutil.which("hipcc")
+FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fvisibility=hidden", "-Xclang",
+         "-target-feature", "-Xclang", "-packed-fp32-ops", "-ffp-contract=off", "-Wno-inline-asm",
+         f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}", "--offload-device-only", "-S"]
+
+
+def kernel_resources(src, outdir):
+    out = os.path.join(outdir, os.path.basename(src) + ".s")
+    subprocess.run([HIPCC, *FLAGS, src, "-o", out], check=True, stdout=subprocess.DEVNULL,
+                   stderr=subprocess.DEVNULL)
+    res, name = {}, None
+    for line in open(out):
+        m = re.match(r"\s+\.name:\s+(\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.match(r"\s+\.vgpr_spill_count:\s+(\d+)", line)
+        if m and name:
+            res[name] = int(m.group(1))
+    return res
+
+
+@pytest.mark.skipif(HIPCC is None, reason="hipcc not installed")
+def test_hot_kernels_do_not_spill():
+    files = [os.path.join(CSRC, f) for f in ("gemm_16b.hip", "gemm_i8.hip", "gemm_f32.hip",
+                                              "gemm_skinny.hip", "gemm_f32_small.hip", "probe.hip")]
+    with tempfile.TemporaryDirectory() as d, concurrent.futures.ThreadPoolExecutor(6) as pool:
+        results = list(pool.map(lambda f: kernel_resources(f, d), files))
+    spills = {k: v for r in results for k, v in r.items()}
+    assert len(spills) > 60          # every template instance was seen
+    for name, n in spills.items():
+        if re.search(r"EpiDequantX4ILb[01]ELb1", name):
+            assert n <= 100, (name, n)     # accumulator-dump variants (a test aid): epilogue only
+        elif "EpiBiasActF32x4" in name:
+            assert n <= 2, (name, n)
+        else:
+            assert n == 0, (name, n)
