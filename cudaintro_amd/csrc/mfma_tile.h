@@ -56,7 +56,6 @@ namespace tile {
 constexpr int BM = 256, BN = 256;
 constexpr int KB = 64;                     // bytes of k per stage, per row
 constexpr int OPERAND_BYTES = 256 * KB;    // 16 KiB, either operand
-constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
 
 typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
 typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
@@ -327,12 +326,11 @@ __device__ __forceinline__ EpiPartialX4 epilogue_of_split(const EpiPartialX4& e,
   return EpiPartialX4{e.base + split * e.split_stride, e.ld, e.split_stride};
 }
 
-// Epi: __device__ void operator()(int64_t row, int64_t col, scalar v0, v1, v2, v3) stores the
-// four consecutive columns col..col+3 of one output row.
+// Epi: an epilogue functor (see epilogues.h): load_row / load_cols / pack / side / out_row.
 //
-// A, B are byte pointers; lda/ldb are in BYTES.  K_bytes = K * ELEM_BYTES is a multiple of
-// 64, M and N multiples of 256, all rows 16-byte aligned (the launcher checks).  KTS = number
-// of 64-byte stages.
+// A, B are byte pointers; lda/ldb are in BYTES.  Any M; N a multiple of 4; all rows 16-byte
+// aligned (tile_shape_ok checks).  KTS = number of 64-byte stages of this workgroup's K
+// range; grid = (tiles, K ranges).
 template <typename Math, int BMODE, int NSTAGES, int MT, typename Epi>
 __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int tiles_m,
                                                            int tiles_n, int KTS,
