@@ -21,8 +21,9 @@
 //         lives at r*128 + ((c ^ ((r >> 1) & 7)) << 4): the 16-byte fragment reads of 32
 //         consecutive rows then spread over all banks.
 // B tile  one of
-//   NK    [256 n][64 B of k]  (weights, k contiguous): 16-byte chunk c of row r at
-//         r*64 + ((c ^ f(r)) << 4), read like A;
+//   NK    (weights, k contiguous) row-major like A, so fetched the same way: pairs
+//         [256 n][128 B of k] of whole lines, two 32 KiB pair slots in the 64 KiB of the
+//         B ring, read like A;
 //   KN16  [32 k][256 n] halves, KN8 [64 k][256 n] bytes (n contiguous, as C = A.B stores
 //         B).  The MFMA wants k contiguous per lane, so fragments come from the transposing
 //         LDS reads ds_read_b64_tr_b16 / _tr_b8: within 16 lanes, lane i supplies the
@@ -37,6 +38,9 @@
 //             stage s+3: 4 instructions of B into the slot stage s-1 just left (every wave
 //             finished reading it before it reached the barrier) and, for odd s, the 8 of
 //             the A pair of stages s+3 and s+4.
+// With N x K weights both operands move as pairs: odd stages issue the B pair and the A pair
+// of stages s+3, s+4 (16 instructions, the B pair into the slot whose last fragments were
+// read in k-step 0 of this stage), even stages none.
 // Fragments are double buffered in registers.  The emitted order is pinned slot by slot
 // with scheduling fences: one MFMA, at most one LDS read, at most one DMA.
 //
@@ -123,6 +127,12 @@ struct BTile<B_NK> : RowMajorDma, HalfPieces {
                                                     int l) {
     const int r = wn * 128 + 32 * j + (l & 31);
     return *reinterpret_cast<const u32x2*>(sb + rowmajor_off(r, 2 * kk + (l >> 5)) + 8 * h);
+  }
+  // the same from a pair tile [256 n][128 B]; par = which stage of the pair
+  static __device__ __forceinline__ u32x2 frag_half_pair(const char* sb, int wn, int j, int par,
+                                                         int kk, int h, int l) {
+    const int r = wn * 128 + 32 * j + (l & 31);
+    return *reinterpret_cast<const u32x2*>(sb + pair_off(r, 4 * par + 2 * kk + (l >> 5)) + 8 * h);
   }
 };
 
@@ -350,8 +360,13 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   constexpr int DIST = NSTAGES - 1;  // stages in flight ahead of the one being multiplied
   constexpr int TILE_M = 64 * MT;    // rows of the macro tile
   static_assert(NSTAGES == 4, "the wait counts below assume three stages in flight");
+  // N x K weights are row-major like A: they too are fetched as whole 128-byte lines, a pair
+  // of stages at a time, into two 32 KiB pair slots (the same 64 KiB as the ring of four
+  // single stages the K x N layouts use).
+  constexpr bool BPAIR = BMODE == B_NK;
   constexpr int DMA_A = 2 * MT;          // per wave and stage pair: A instructions of 1 KiB
-  constexpr int DMA_B = 4;               // per wave and stage: B instructions
+  constexpr int DMA_B = BPAIR ? 8 : 4;   // per wave: B instructions per stage pair / per stage
+  constexpr int BPAIR_BYTES = 256 * 128;
   constexpr int APAIR_BYTES = TILE_M * 128;
   constexpr int B_RING = NSTAGES * OPERAND_BYTES;   // B slots first, then three A pair slots
   typedef RowPairDmaT<MT> ADma;
@@ -394,11 +409,21 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   }
   const int last_pair = (KTS - 1) >> 1;
   const bool odd_kts = KTS & 1;
-  uint32_t a_voff[DMA_A], b_voff[4];
+  uint32_t b_hi = 0;  // the same for the rows of N x K weights
+  if (BPAIR) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int r = 64 * w + 8 * i + (l >> 3);
+      b_hi |= (uint32_t)((((l & 7) ^ pair_swz(r)) >> 2) & 1) << i;
+    }
+  }
+  uint32_t a_voff[DMA_A], b_voff[DMA_B];
 #pragma unroll
   for (int i = 0; i < DMA_A; ++i) a_voff[i] = (uint32_t)ADma::dma_src(w, i, l, lda, a_last);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) b_voff[i] = (uint32_t)BT::dma_src(w, i, l, ldb, b_last);
+  for (int i = 0; i < DMA_B; ++i)
+    b_voff[i] = BPAIR ? (uint32_t)RowPairDmaT<4>::dma_src(w, i, l, ldb, b_last)
+                      : (uint32_t)BT::dma_src(w, i, l, ldb, b_last);
 
   // The DMA instructions are written as asm so that the compiler's wait-count insertion does
   // not know them: it would otherwise make every later LDS read it cannot tell apart (the
@@ -412,20 +437,28 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
                  : "s"(lds_dst), "v"(src)
                  : "m0");
   };
-  // d < 4: B instruction d of stage `st` into B slot `slot`; d >= 4: A instruction d - 4 of
-  // the stage pair st / 2 into pair slot `pslot`.  Past the last stage the last one is fetched
+  // d < DMA_B: B instruction d of stage `st` (of its stage pair, for N x K weights) into B
+  // slot `slot`; above: A instruction d - DMA_B of the stage pair st / 2 into pair slot `pslot`.  Past the last stage the last one is fetched
   // again (into slots nobody reads any more), which keeps the number of outstanding
   // instructions, and so the vmcnt waits, uniform.
   auto dma_piece = [&](int st, int slot, int pslot, int d) {
     st = st < KTS ? st : KTS - 1;
-    if (d < 4)
-      dma16(b_tile + (int64_t)st * b_kstep + b_voff[d],
-            lds_base + slot * OPERAND_BYTES + BT::dma_lds(w, d));
-    else {
-      uint32_t off = a_voff[d - 4];
-      if (odd_kts && (st >> 1) == last_pair) off -= ((a_hi >> (d - 4)) & 1u) << 6;
+    const bool tail_pair = odd_kts && (st >> 1) == last_pair;
+    if (d < DMA_B) {
+      if (BPAIR) {
+        uint32_t off = b_voff[d];
+        if (tail_pair) off -= ((b_hi >> d) & 1u) << 6;
+        dma16(b_tile + (int64_t)(st >> 1) * 128 + off,
+              lds_base + slot * BPAIR_BYTES + RowPairDmaT<4>::dma_lds(w, d));
+      } else {
+        dma16(b_tile + (int64_t)st * b_kstep + b_voff[d],
+              lds_base + slot * OPERAND_BYTES + BT::dma_lds(w, d));
+      }
+    } else {
+      uint32_t off = a_voff[d - DMA_B];
+      if (tail_pair) off -= ((a_hi >> (d - DMA_B)) & 1u) << 6;
       dma16(a_tile + (int64_t)(st >> 1) * 128 + off,
-            lds_base + B_RING + pslot * APAIR_BYTES + ADma::dma_lds(w, d - 4));
+            lds_base + B_RING + pslot * APAIR_BYTES + ADma::dma_lds(w, d - DMA_B));
     }
   };
 
@@ -447,6 +480,9 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
     if (r < MT)
       f.a[r] = *reinterpret_cast<const u32x4*>(
           lds + B_RING + pslot * APAIR_BYTES + pair_off(a_frag_row + 32 * r, 4 * par + 2 * kk + g));
+    else if constexpr (BPAIR)
+      f.b[r - MT] = BT::frag_half_pair(lds + slot * BPAIR_BYTES, wn, (r - MT) >> 1, par, kk,
+                                       (r - MT) & 1, l);
     else
       f.b[r - MT] = read_b_piece<BMODE>(lds + slot * OPERAND_BYTES, wn, r - MT, kk, l);
   };
@@ -474,29 +510,35 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
     __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
   };
 
-  // prologue, in the order the main loop keeps: B[0], A pair 0, B[1], B[2], A pair 1; stage
-  // 0 landed; first fragments in registers
+  // prologue, in the order the main loop keeps -- single B stages: B[0], A pair 0, B[1], B[2],
+  // A pair 1; B pairs: B pair 0, A pair 0, B pair 1, A pair 1 -- then stage 0 landed and the
+  // first fragments in registers
 #pragma unroll
   for (int d = 0; d < DMA_B + DMA_A; ++d) dma_piece(0, 0, 0, d);
+  if (!BPAIR) {
 #pragma unroll
-  for (int d = 0; d < DMA_B; ++d) dma_piece(1, 1, 0, d);
+    for (int d = 0; d < DMA_B; ++d) dma_piece(1, 1, 0, d);
+  }
 #pragma unroll
-  for (int d = 0; d < DMA_B + DMA_A; ++d) dma_piece(2, 2, 1, d);
-  wait_vmcnt(std::integral_constant<int, 2 * DMA_B + DMA_A>{});
+  for (int d = 0; d < DMA_B + DMA_A; ++d) dma_piece(2, BPAIR ? 1 : 2, 1, d);
+  wait_vmcnt(std::integral_constant<int, BPAIR ? DMA_B + DMA_A : 2 * DMA_B + DMA_A>{});
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int r = 0; r < NREAD; ++r) read_piece(f0, 0, 0, 0, 0, r);
-  // B ring slots of the stage being multiplied, of the next one, and of the one the DMA
-  // fills (wave-uniform scalars, advanced modulo NSTAGES each stage); the three A pair slots
-  // likewise, advanced every second stage.
+  // Single B stages: ring slots of the stage being multiplied, of the next one, and of the one
+  // the DMA fills (wave-uniform scalars, advanced modulo NSTAGES each stage).  B pairs: the
+  // slot of the pair being multiplied and the other one, swapped every second stage; the DMA
+  // refills the current one once its last fragments are in registers.  The three A pair slots
+  // advance every second stage.
   int slot = 0, next_slot = 1, dma_slot = DIST;
   int pslot = 0, next_pslot = 1, dma_pslot = 2;
-  // One stage; PAR = its parity.  Even stages issue B[s+3] only; odd stages B[s+3] and the A
-  // pair of stages s+3, s+4.
+  // One stage; PAR = its parity.  Single B stages: even stages issue B[s+3] only, odd stages
+  // B[s+3] and the A pair of stages s+3, s+4.  B pairs: odd stages issue both pairs of stages
+  // s+3, s+4, even stages nothing.
   auto stage = [&](int s, auto par_const) {
     constexpr int PAR = decltype(par_const)::value;
-    constexpr int NDMA = PAR ? DMA_B + DMA_A : DMA_B;
+    constexpr int NDMA = BPAIR ? (PAR ? DMA_B + DMA_A : 0) : (PAR ? DMA_B + DMA_A : DMA_B);
 #pragma unroll
     for (int sl = 0; sl < NMFMA; ++sl) {
       mfma_piece(f0, sl);
@@ -505,9 +547,19 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
         if (r < NREAD) read_piece(f1, slot, pslot, PAR, 1, r);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // stage s+1 landed for this wave.  Still in flight, in issue order after what stage s+1
-    // needs: even s: B[s+2] and the A pair (s+2, s+3); odd s: B[s+2].
-    wait_vmcnt(std::integral_constant<int, PAR ? DMA_B : DMA_B + DMA_A>{});
+    if (BPAIR) {
+      // Odd stage: the next pair (issued two stages ago, nothing newer in flight) landed;
+      // this wave's last reads of the current B pair slot are complete before any wave
+      // refills it after the barrier.  Even stage: stage s+1 is in the pair already landed.
+      if (PAR) {
+        wait_vmcnt(std::integral_constant<int, 0>{});
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+    } else {
+      // stage s+1 landed for this wave.  Still in flight, in issue order after what stage
+      // s+1 needs: even s: B[s+2] and the A pair (s+2, s+3); odd s: B[s+2].
+      wait_vmcnt(std::integral_constant<int, PAR ? DMA_B : DMA_B + DMA_A>{});
+    }
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -515,15 +567,25 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
       mfma_piece(f1, sl);
 #pragma unroll
       for (int r = sl * READS_PER_SLOT; r < (sl + 1) * READS_PER_SLOT; ++r)
-        if (r < NREAD) read_piece(f0, next_slot, PAR ? next_pslot : pslot, PAR ^ 1, 0, r);
+        if (r < NREAD)
+          read_piece(f0, BPAIR ? (PAR ? next_slot : slot) : next_slot, PAR ? next_pslot : pslot,
+                     PAR ^ 1, 0, r);
 #pragma unroll
       for (int d = sl * DMA_PER_SLOT; d < (sl + 1) * DMA_PER_SLOT; ++d)
-        if (d < NDMA) dma_piece(s + DIST, dma_slot, dma_pslot, d);
+        if (d < NDMA) dma_piece(s + DIST, BPAIR ? slot : dma_slot, dma_pslot, d);
       __builtin_amdgcn_sched_barrier(0);
     }
-    slot = next_slot;
-    next_slot = next_slot + 1 == NSTAGES ? 0 : next_slot + 1;
-    dma_slot = dma_slot + 1 == NSTAGES ? 0 : dma_slot + 1;
+    if (BPAIR) {
+      if (PAR) {
+        const int tmp = slot;
+        slot = next_slot;
+        next_slot = tmp;
+      }
+    } else {
+      slot = next_slot;
+      next_slot = next_slot + 1 == NSTAGES ? 0 : next_slot + 1;
+      dma_slot = dma_slot + 1 == NSTAGES ? 0 : dma_slot + 1;
+    }
     if (PAR) {
       pslot = next_pslot;
       next_pslot = next_pslot + 1 == 3 ? 0 : next_pslot + 1;
