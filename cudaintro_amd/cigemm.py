@@ -68,6 +68,7 @@ SIGNATURES = {
     "cigemmGetLastErrorString": (C.c_char_p, [_vp]),
     "cigemmGetVersion": (_ci, []),
     "cigemmGetLastKernelName": (C.c_char_p, [_vp]),
+    "cigemmGetLastPlan": (C.c_int, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "cigemm_matrixMulTiled": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
     "cigemm_matrixMulMatrixCores": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
     "cigemm_matrixMulMatrixCoresBfloat16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
@@ -182,6 +183,14 @@ class Handle:
     @property
     def last_kernel(self) -> str:
         return self.lib.cigemmGetLastKernelName(self._h).decode()
+
+    @property
+    def last_plan(self):
+        """(tile rows, K ranges) of the last GEMM when the LDS-tiled kernel ran, else (0, 0)."""
+        rows, splits = C.c_int(0), C.c_int(0)
+        self._check(self.lib.cigemmGetLastPlan(self._h, C.byref(rows), C.byref(splits)),
+                    "cigemmGetLastPlan")
+        return rows.value, splits.value
 
     # -- GEMMs ------------------------------------------------------------------------------
     @staticmethod

@@ -35,6 +35,8 @@ bool valid(cigemmHandle_t h) { return h && h->magic == kCtxMagic; }
 cigemmStatus_t check_gemm_args(cigemmHandle_t h, const char* name, int64_t M, int64_t N,
                                int64_t K, const void* A, int64_t lda, const void* B,
                                int64_t ldb, int64_t b_cols, const void* C, int64_t ldc) {
+  h->last_tile_rows = 0;  // set again by the tile kernel's launcher
+  h->last_k_splits = 0;
   if (M < 0 || N < 0 || K < 0)
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: negative dimension (M=%lld N=%lld K=%lld)",
                 name, (long long)M, (long long)N, (long long)K);
@@ -88,6 +90,8 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->num_cus = prop.multiProcessorCount;
   ctx->stream = nullptr;
   ctx->last_kernel = "";
+  ctx->last_tile_rows = 0;
+  ctx->last_k_splits = 0;
   ctx->algo = CIGEMM_ALGO_DEFAULT;
   ctx->last_error[0] = '\0';
   ctx->ws_partial_bytes = (size_t)64 << 20;
@@ -145,6 +149,13 @@ const char* cigemmGetLastErrorString(cigemmHandle_t h) { return valid(h) ? h->la
 int cigemmGetVersion(void) { return 100; }
 
 const char* cigemmGetLastKernelName(cigemmHandle_t h) { return valid(h) ? h->last_kernel : ""; }
+
+cigemmStatus_t cigemmGetLastPlan(cigemmHandle_t h, int* tile_rows, int* k_splits) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if (tile_rows) *tile_rows = h->last_tile_rows;
+  if (k_splits) *k_splits = h->last_k_splits;
+  return CIGEMM_STATUS_SUCCESS;
+}
 
 cigemmStatus_t cigemmSetAlgo(cigemmHandle_t h, cigemmAlgo_t algo) {
   if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;

@@ -16,6 +16,8 @@ struct cigemmContext {
   int num_cus;
   hipStream_t stream;
   const char* last_kernel;
+  int last_tile_rows;  // rows of the output tile of the last tile-kernel launch, 0 otherwise
+  int last_k_splits;   // K ranges of that launch
   int algo;  // cigemmAlgo_t; -1 = choose by shape
   // Device scratch of the split-K kernels, allocated once at create: `ws_partial_bytes` of
   // partial sums followed by `ws_counter_bytes` of arrival counters (zero between calls).

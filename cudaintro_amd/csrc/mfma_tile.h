@@ -3,8 +3,8 @@
 // Workgroup = 256 lanes = 4 waves (2 x 2); macro tile 256 (m) x 256 (n); k is consumed in
 // stages of 64 BYTES per row (32 halves, 64 int8 or 16 floats) = two MFMA k-steps.  Each wave
 // owns a 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulators per lane (the AGPR
-// file); one wave per SIMD.  The tile height is a template parameter (MT = 4, 2 or 1 row
-// tiles per wave: 256, 128 or 64 rows) so that small or awkward M still fill the chip; the
+// file); one wave per SIMD.  The tile height is a template parameter (MT = 4, 3, 2 or 1 row
+// tiles per wave: 256, 192, 128 or 64 rows) so that small or awkward M still fill the chip; the
 // text below describes MT = 4.  Both operand tiles of a stage are 16 KiB.  B stages form a
 // ring of 4 slots in LDS (64 KiB), three of them in flight ahead of the one being multiplied:
 // HBM/L2 latency here is of the order of a microsecond, two to three stage times.  A is
@@ -674,6 +674,8 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
     attr_device = ctx->device;
   }
   const int tiles_m = (int)((M + 64 * MT - 1) / (64 * MT)), tiles_n = (int)((N + BN - 1) / BN);
+  ctx->last_tile_rows = 64 * MT;
+  ctx->last_k_splits = splits;
   const int64_t kts = K_bytes / KB / splits;  // stages per K range
   const int64_t a_step = kts * KB;
   const int64_t b_step = BMODE == B_NK ? kts * KB : kts * (KB / Math::ELEM_BYTES) * ldb_bytes;
@@ -727,16 +729,25 @@ struct SmallPlan {
   int mt;
   int splits;
 };
+// Cost of one tile of 64*mt rows, in units of a quarter of the 256-row tile's: a fixed part
+// (the B panel is fetched whatever the height) plus a part per 64 rows; the fixed part weighs
+// more when B streams from HBM than when it sits in the L2 / Infinity Cache.  One round of
+// 256 tiles, N = 4096, K = 1024..4096, 16-bit and int8: 4.0 / 3.1-3.2 / 2.3 / 1.6-1.8;
+// 2 x 32 tiles over 8192 x 8192 weights: 4.0 / 3.0-3.5 / 2.5 / 1.9-2.3.
+inline double tile_cost_units(int mt, bool streamed) {
+  return streamed ? 1.2 + 0.7 * mt : 0.8 + 0.8 * mt;
+}
+
 inline SmallPlan plan_small(const cigemmContext* ctx, int64_t M, int64_t N, int64_t kts,
                             double sm_us, int64_t b_bytes) {
   const bool streamed = b_bytes > (16LL << 20);
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
   SmallPlan best{0, 1};
   double best_us = 1e30;
-  for (int mt : {4, 2, 1}) {
-    if (mt > 1 && 64 * (mt / 2) >= M) continue;  // half the height already covers M
+  for (int mt : {4, 3, 2, 1}) {
+    if (mt > 1 && 64 * (mt - 1) >= M) continue;  // the next lower height already covers M
     const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + BN - 1) / BN);
-    const double per_tile = mt == 4 ? 4.0 : mt == 2 ? (streamed ? 2.5 : 2.24) : (streamed ? 1.7 : 1.3);
+    const double per_tile = tile_cost_units(mt, streamed);
     for (int sp = 1; sp <= 16; sp *= 2) {
       if (sp > 1) {
         if (!ctx->workspace || kts % sp || kts / sp < 8) break;
@@ -758,13 +769,12 @@ inline SmallPlan plan_small(const cigemmContext* ctx, int64_t M, int64_t N, int6
 // workgroups times the cost of one tile; shorter tiles re-read B more often per flop.
 inline double tile_plan_cost(int64_t M, int64_t N, int mt, int cus) {
   const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + BN - 1) / BN);
-  const double per_tile = mt == 4 ? 4.0 : mt == 2 ? 2.0 * 1.12 : 1.0 * 1.3;
-  return (double)((tiles + cus - 1) / cus) * per_tile;
+  return (double)((tiles + cus - 1) / cus) * tile_cost_units(mt, false);
 }
 inline int best_mt(int64_t M, int64_t N, int cus, double* cost = nullptr) {
   int best = 0;
   double bc = 1e30;
-  for (int mt : {4, 2, 1}) {
+  for (int mt : {4, 3, 2, 1}) {
     const double c = tile_plan_cost(M, N, mt, cus);
     if (c < bc) {
       bc = c;
@@ -781,6 +791,8 @@ void launch_tile_any_mt(cigemmContext* ctx, int mt, int64_t M, int64_t N, int64_
                         const Epi& epi, int splits = 1) {
   if (mt == 4)
     launch_tile_mt<Math, BMODE, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
+  else if (mt == 3)
+    launch_tile_mt<Math, BMODE, 3>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
   else if (mt == 2)
     launch_tile_mt<Math, BMODE, 2>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
   else

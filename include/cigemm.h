@@ -94,6 +94,13 @@ CIGEMM_API int cigemmGetVersion(void);
  * (for tests and profiles), e.g. "bf16_mfma_256x256x32_ring4". */
 CIGEMM_API const char* cigemmGetLastKernelName(cigemmHandle_t handle);
 
+/* Plan of the last successful GEMM call on this handle, for tests and profiles: rows of the
+ * output tile (256, 192, 128 or 64; with two launches, of the second) and number of K ranges
+ * when the LDS-tiled matrix-core kernel ran, 0 and 0 when another family did.  Either pointer
+ * may be null.  No counterpart in the reference: cuBLAS does not report its heuristics'
+ * choice (quantization/GEMM_bf16.cu:51-56). */
+CIGEMM_API cigemmStatus_t cigemmGetLastPlan(cigemmHandle_t handle, int* tile_rows, int* k_splits);
+
 /* Kernel family selection: the counterpart of cublasGemmEx's `algo` argument (the reference
  * passes CUBLAS_GEMM_DEFAULT_TENSOR_OP, quantization/GEMM_bf16.cu:56), kept on the handle.
  * DEFAULT lets the library choose by shape.  A specific family restricts every following GEMM
