@@ -306,12 +306,12 @@ def main():
         # What the matrix cores sustain with no memory traffic at all, at the clock the chip
         # holds under that load, on constant and on random operand bits.
         probe = {}
-        for kind in ("bf16", "f16", "i8"):
+        for kind in ("bf16", "f16", "i8", "f32"):
             for rnd in (False, True):
                 ops_box = [0]
 
                 def fnp():
-                    ops_box[0] = handle.probe_mfma(kind, rnd, 20000)
+                    ops_box[0] = handle.probe_mfma(kind, rnd, 5000 if kind == "f32" else 20000)
                 w, e = time_calls(torch, fnp, 20, 10)
                 probe[f"{kind}_{'random' if rnd else 'constant'}_bits"] = ops_box[0] * 20 / e / 1e12
         mfma_probe.update(probe)

@@ -238,7 +238,8 @@ class Handle:
     def probe_mfma(self, kind: str, random_bits: bool, iters: int) -> int:
         """Launch the register-resident matrix-core loop; returns the operations it performs."""
         ops = C.c_int64(0)
-        k = {"bf16": 0, "f16": 1, "i8": 2, "bf16_16x16": 3, "f16_16x16": 4, "i8_16x16": 5}[kind]
+        k = {"bf16": 0, "f16": 1, "i8": 2, "bf16_16x16": 3, "f16_16x16": 4, "i8_16x16": 5,
+             "f32": 6}[kind]
         self._check(self.lib.cigemm_probe_mfma(self._h, k, int(random_bits), iters, C.byref(ops)),
                     "cigemm_probe_mfma")
         return ops.value

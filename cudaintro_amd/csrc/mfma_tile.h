@@ -378,6 +378,10 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
 
   int tm, tn;
   tile_of_workgroup(tiles_m, tiles_n, tm, tn);
+  // (the divisions above run on the vector unit: tell the compiler the results are uniform,
+  // so that everything derived from them, the DMA base addresses above all, stays scalar)
+  tm = __builtin_amdgcn_readfirstlane(tm);
+  tn = __builtin_amdgcn_readfirstlane(tn);
   const int64_t m0 = (int64_t)tm * TILE_M, n0 = (int64_t)tn * BN;
 
   // ---- DMA sources: uniform tile origin + per-lane byte offsets ------------------------------
@@ -429,38 +433,47 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   // not know them: it would otherwise make every later LDS read it cannot tell apart (the
   // transposing reads) wait for all outstanding DMA.  Completion is waited for by hand
   // (vmcnt) before the barrier that publishes a stage.  M0 carries the wave-uniform LDS
-  // destination; lane l's 16 bytes land at M0 + 16 l.
+  // destination; lane l's 16 bytes land at M0 + 16 l.  The source is a scalar base (tile origin
+  // + stage, advanced on the scalar unit) plus a loop-invariant 32-bit lane offset: no vector
+  // ALU work per instruction (on this chip every vector instruction between two matrix
+  // instructions delays the second, by about a cycle under the 16-bit and int8 ones and by
+  // ten and more under the fp32 one, which runs on the vector ALU's own multipliers).
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
-  auto dma16 = [&](const char* src, uint32_t lds_dst) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+  auto dma16 = [&](const char* base, uint32_t voff, uint32_t lds_dst) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
-                 : "s"(lds_dst), "v"(src)
+                 : "s"(lds_dst), "v"(voff), "s"(base)
                  : "m0");
   };
   // d < DMA_B: B instruction d of stage `st` (of its stage pair, for N x K weights) into B
   // slot `slot`; above: A instruction d - DMA_B of the stage pair st / 2 into pair slot `pslot`.  Past the last stage the last one is fetched
   // again (into slots nobody reads any more), which keeps the number of outstanding
   // instructions, and so the vmcnt waits, uniform.
-  auto dma_piece = [&](int st, int slot, int pslot, int d) {
-    st = st < KTS ? st : KTS - 1;
-    const bool tail_pair = odd_kts && (st >> 1) == last_pair;
+  // `steady_const`: the caller guarantees st < KTS and a pair that is not the odd tail, so
+  // that no per-lane arithmetic is left: the uniform part of the address is a scalar base.
+  auto dma_piece = [&](int st, int slot, int pslot, int d, auto steady_const) {
+    constexpr bool STEADY = decltype(steady_const)::value;
+    if (!STEADY) st = st < KTS ? st : KTS - 1;
+    const bool tail_pair = !STEADY && odd_kts && (st >> 1) == last_pair;
     if (d < DMA_B) {
       if (BPAIR) {
         uint32_t off = b_voff[d];
         if (tail_pair) off -= ((b_hi >> d) & 1u) << 6;
-        dma16(b_tile + (int64_t)(st >> 1) * 128 + off,
+        dma16(b_tile + (int64_t)(st >> 1) * 128, off,
               lds_base + slot * BPAIR_BYTES + RowPairDmaT<4>::dma_lds(w, d));
       } else {
-        dma16(b_tile + (int64_t)st * b_kstep + b_voff[d],
+        dma16(b_tile + (int64_t)st * b_kstep, b_voff[d],
               lds_base + slot * OPERAND_BYTES + BT::dma_lds(w, d));
       }
     } else {
       uint32_t off = a_voff[d - DMA_B];
       if (tail_pair) off -= ((a_hi >> (d - DMA_B)) & 1u) << 6;
-      dma16(a_tile + (int64_t)(st >> 1) * 128 + off,
+      dma16(a_tile + (int64_t)(st >> 1) * 128, off,
             lds_base + B_RING + pslot * APAIR_BYTES + ADma::dma_lds(w, d - DMA_B));
     }
   };
+  typedef std::integral_constant<bool, true> steady_t;
+  typedef std::integral_constant<bool, false> drain_t;
 
   const int a_frag_row = wm * 32 * MT + (l & 31);
   const int g = l >> 5;
@@ -514,13 +527,13 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   // A pair 1; B pairs: B pair 0, A pair 0, B pair 1, A pair 1 -- then stage 0 landed and the
   // first fragments in registers
 #pragma unroll
-  for (int d = 0; d < DMA_B + DMA_A; ++d) dma_piece(0, 0, 0, d);
+  for (int d = 0; d < DMA_B + DMA_A; ++d) dma_piece(0, 0, 0, d, drain_t{});
   if (!BPAIR) {
 #pragma unroll
-    for (int d = 0; d < DMA_B; ++d) dma_piece(1, 1, 0, d);
+    for (int d = 0; d < DMA_B; ++d) dma_piece(1, 1, 0, d, drain_t{});
   }
 #pragma unroll
-  for (int d = 0; d < DMA_B + DMA_A; ++d) dma_piece(2, BPAIR ? 1 : 2, 1, d);
+  for (int d = 0; d < DMA_B + DMA_A; ++d) dma_piece(2, BPAIR ? 1 : 2, 1, d, drain_t{});
   wait_vmcnt(std::integral_constant<int, BPAIR ? DMA_B + DMA_A : 2 * DMA_B + DMA_A>{});
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
@@ -536,7 +549,7 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   // One stage; PAR = its parity.  Single B stages: even stages issue B[s+3] only, odd stages
   // B[s+3] and the A pair of stages s+3, s+4.  B pairs: odd stages issue both pairs of stages
   // s+3, s+4, even stages nothing.
-  auto stage = [&](int s, auto par_const) {
+  auto stage = [&](int s, auto par_const, auto steady_const) {
     constexpr int PAR = decltype(par_const)::value;
     constexpr int NDMA = BPAIR ? (PAR ? DMA_B + DMA_A : 0) : (PAR ? DMA_B + DMA_A : DMA_B);
 #pragma unroll
@@ -572,7 +585,7 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
                      PAR ^ 1, 0, r);
 #pragma unroll
       for (int d = sl * DMA_PER_SLOT; d < (sl + 1) * DMA_PER_SLOT; ++d)
-        if (d < NDMA) dma_piece(s + DIST, BPAIR ? slot : dma_slot, dma_pslot, d);
+        if (d < NDMA) dma_piece(s + DIST, BPAIR ? slot : dma_slot, dma_pslot, d, steady_const);
       __builtin_amdgcn_sched_barrier(0);
     }
     if (BPAIR) {
@@ -592,11 +605,17 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
       dma_pslot = dma_pslot + 1 == 3 ? 0 : dma_pslot + 1;
     }
   };
-  for (int s = 0; s + 1 < KTS; s += 2) {
-    stage(s, std::integral_constant<int, 0>{});
-    stage(s + 1, std::integral_constant<int, 1>{});
+  // Steady part: every stage the DMA reaches (up to s + 5) exists and is not the odd tail.
+  int s = 0;
+  for (; s + 5 < KTS; s += 2) {
+    stage(s, std::integral_constant<int, 0>{}, steady_t{});
+    stage(s + 1, std::integral_constant<int, 1>{}, steady_t{});
   }
-  if (KTS & 1) stage(KTS - 1, std::integral_constant<int, 0>{});  // odd stage count: the last one
+  for (; s + 1 < KTS; s += 2) {
+    stage(s, std::integral_constant<int, 0>{}, drain_t{});
+    stage(s + 1, std::integral_constant<int, 1>{}, drain_t{});
+  }
+  if (KTS & 1) stage(KTS - 1, std::integral_constant<int, 0>{}, drain_t{});  // odd stage count: the last one
   wait_vmcnt(std::integral_constant<int, 0>{});  // no DMA outlives the main loop
   __syncthreads();  // ... for any wave, and every wave is done reading the ring
 
@@ -860,7 +879,7 @@ bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
 // b_kn = B is K x N).  M is free; K must fill whole 64-byte stages (nothing pads k with
 // zeros); N must keep 16-byte pieces whole, on the input side (K x N rows) and on the output
 // side (the caller checks its output type).  Per-lane DMA offsets are 32-bit: 256 rows of
-// either operand must span less than 4 GiB.
+// either operand must span less than 2 GiB.
 inline bool tile_shape_ok(int64_t M, int64_t N, int64_t K, int elem, const void* A, int64_t lda,
                           const void* B, int64_t ldb, bool b_kn) {
   if (M <= 0 || N <= 0 || K <= 0) return false;
@@ -870,7 +889,7 @@ inline bool tile_shape_ok(int64_t M, int64_t N, int64_t K, int elem, const void*
   if ((lda * elem) % 16 || (ldb * elem) % 16) return false;
   if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return false;
   if (((M + 63) / 64) * ((N + BN - 1) / BN) > 2147483647LL) return false;
-  if (lda * elem * 256 >= (1LL << 32) || ldb * elem * 256 >= (1LL << 32)) return false;
+  if (lda * elem * 256 >= (1LL << 31) || ldb * elem * 256 >= (1LL << 31)) return false;
   return true;
 }
 

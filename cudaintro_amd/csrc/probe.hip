@@ -15,7 +15,7 @@ __device__ __forceinline__ uint32_t mix32(uint32_t x) {
 }
 
 // KIND 0: bf16 32x32x16, 1: f16 32x32x16, 2: int8 32x32x32, 3: bf16 16x16x32, 4: f16 16x16x32,
-// 5: int8 16x16x64.
+// 5: int8 16x16x64, 6: fp32 32x32x2.
 template <int KIND>
 __global__ __launch_bounds__(256, 1) void mfma_probe_kernel(float* __restrict__ out, int iters,
                                                             int random_bits) {
@@ -35,6 +35,9 @@ __global__ __launch_bounds__(256, 1) void mfma_probe_kernel(float* __restrict__ 
       } else if (KIND == 1 || KIND == 4) {  // +-[1,2) in fp16
         xa = (xa & 0x83ff83ffu) | 0x3c003c00u;
         xb = (xb & 0x83ff83ffu) | 0x3c003c00u;
+      } else if (KIND == 6) {  // +-[1,2) in fp32
+        xa = (xa & 0x807fffffu) | 0x3f800000u;
+        xb = (xb & 0x807fffffu) | 0x3f800000u;
       } else if (!random_bits) {
         xa = xb = 0x01010101u;
       }
@@ -78,6 +81,9 @@ __global__ __launch_bounds__(256, 1) void mfma_probe_kernel(float* __restrict__ 
       else if (KIND == 4)
         facc4[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, x),
                                                           __builtin_bit_cast(f16x8, y), facc4[i], 0, 0, 0);
+      else if (KIND == 6)
+        facc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, x[i & 3 ^ 1]),
+                                                       __builtin_bit_cast(float, y[i & 3]), facc[i], 0, 0, 0);
       else
         iacc4[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, x),
                                                          __builtin_bit_cast(i32x4, y), iacc4[i], 0, 0, 0);
@@ -99,7 +105,7 @@ using namespace cig;
 extern "C" cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t h, int kind, int random_bits, int iters,
                                             int64_t* ops_per_launch) {
   if (!h || h->magic != kCtxMagic) return CIGEMM_STATUS_NOT_INITIALIZED;
-  if (kind < 0 || kind > 5 || iters <= 0 || iters > (1 << 24))
+  if (kind < 0 || kind > 6 || iters <= 0 || iters > (1 << 24))
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "cigemm_probe_mfma: kind %d, iters %d", kind, iters);
   const int grid = h->num_cus > 0 ? h->num_cus : 256;
   if (!h->workspace || (size_t)grid * 256 * sizeof(float) > h->ws_partial_bytes)
@@ -115,11 +121,13 @@ extern "C" cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t h, int kind, int rand
     hipLaunchKernelGGL(mfma_probe_kernel<3>, dim3(grid), dim3(256), 0, h->stream, out, iters, random_bits);
   else if (kind == 4)
     hipLaunchKernelGGL(mfma_probe_kernel<4>, dim3(grid), dim3(256), 0, h->stream, out, iters, random_bits);
-  else
+  else if (kind == 5)
     hipLaunchKernelGGL(mfma_probe_kernel<5>, dim3(grid), dim3(256), 0, h->stream, out, iters, random_bits);
+  else
+    hipLaunchKernelGGL(mfma_probe_kernel<6>, dim3(grid), dim3(256), 0, h->stream, out, iters, random_bits);
   if (ops_per_launch)
     *ops_per_launch = (int64_t)grid * 4 * (int64_t)iters * PROBE_UNROLL *
-                      (kind == 2 ? 65536 : kind == 5 ? 32768 : kind >= 3 ? 16384 : 32768);
+                      (kind == 2 ? 65536 : kind == 6 ? 4096 : kind == 5 ? 32768 : kind >= 3 ? 16384 : 32768);
   h->last_kernel = "mfma_probe";
   return check_launch(h, "cigemm_probe_mfma");
 }

@@ -203,7 +203,7 @@ CIGEMM_API cigemmStatus_t cigemm_matrixMulMatrixCoresBfloat16(cigemmHandle_t han
 /* No counterpart in the reference.  Launches a register-resident matrix-core loop (no memory
  * traffic inside the loop) on every compute unit of the handle's device, on the handle's
  * stream: kind 0 = bf16 32x32x16, 1 = fp16 32x32x16, 2 = int8 32x32x32, 3 = bf16 16x16x32,
- * 4 = fp16 16x16x32, 5 = int8 16x16x64; random_bits 0 =
+ * 4 = fp16 16x16x32, 5 = int8 16x16x64, 6 = fp32 32x32x2; random_bits 0 =
  * constant operands, 1 = pseudo-random operand bits (sustained clocks depend on the data);
  * `iters` loop trips of 12 instructions per wave.  *ops_per_launch receives 2.M.N.K summed
  * over all instructions, for the caller to divide by the time it measures. */

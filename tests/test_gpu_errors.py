@@ -115,7 +115,8 @@ def test_matrix_core_probe(handle, torch_gpu):
     torch_gpu.cuda.synchronize()
     assert handle.last_kernel == "mfma_probe"
     n = ctypes.c_int64(0)
-    assert handle.lib.cigemm_probe_mfma(handle.raw, 6, 0, 10, ctypes.byref(n)) == Status.INVALID_VALUE
+    assert handle.probe_mfma("f32", True, 10) == ops // 8
+    assert handle.lib.cigemm_probe_mfma(handle.raw, 7, 0, 10, ctypes.byref(n)) == Status.INVALID_VALUE
     assert handle.lib.cigemm_probe_mfma(handle.raw, 0, 0, 0, ctypes.byref(n)) == Status.INVALID_VALUE
     assert handle.lib.cigemm_probe_mfma(handle.raw, 0, 0, 10, None) == Status.SUCCESS
     torch_gpu.cuda.synchronize()
