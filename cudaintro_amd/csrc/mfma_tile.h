@@ -23,7 +23,8 @@
 // B tile  one of
 //   NK    (weights, k contiguous) row-major like A, so fetched the same way: pairs
 //         [256 n][128 B of k] of whole lines, two 32 KiB pair slots in the 64 KiB of the
-//         B ring, read like A;
+//         B ring, read like A (one 16-byte read per fragment: 8-byte half reads of this layout
+//         would collide two ways, a wave's 32 rows falling on 16 bank groups);
 //   KN16  [32 k][256 n] halves, KN8 [64 k][256 n] bytes (n contiguous, as C = A.B stores
 //         B).  The MFMA wants k contiguous per lane, so fragments come from the transposing
 //         LDS reads ds_read_b64_tr_b16 / _tr_b8: within 16 lanes, lane i supplies the
@@ -128,11 +129,12 @@ struct BTile<B_NK> : RowMajorDma, HalfPieces {
     const int r = wn * 128 + 32 * j + (l & 31);
     return *reinterpret_cast<const u32x2*>(sb + rowmajor_off(r, 2 * kk + (l >> 5)) + 8 * h);
   }
-  // the same from a pair tile [256 n][128 B]; par = which stage of the pair
-  static __device__ __forceinline__ u32x2 frag_half_pair(const char* sb, int wn, int j, int par,
-                                                         int kk, int h, int l) {
+  // whole fragment (16 bytes) of column tile j from a pair tile [256 n][128 B], read like an
+  // A fragment; par = which stage of the pair
+  static __device__ __forceinline__ u32x4 frag_pair(const char* sb, int wn, int j, int par, int kk,
+                                                    int l) {
     const int r = wn * 128 + 32 * j + (l & 31);
-    return *reinterpret_cast<const u32x2*>(sb + pair_off(r, 4 * par + 2 * kk + (l >> 5)) + 8 * h);
+    return *reinterpret_cast<const u32x4*>(sb + pair_off(r, 4 * par + 2 * kk + (l >> 5)));
   }
 };
 
@@ -479,13 +481,15 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   const int g = l >> 5;
 
   // One k-step's operands: MT A fragments (16 B each) and the pieces of the 4 B fragments.
-  constexpr int NREAD = MT + BT::NREADS;               // LDS reads per k-step
+  // N x K pairs: one 16-byte read per B fragment, kept behind the A fragments in Frags::a
+  constexpr int NREAD_B = BPAIR ? 4 : BT::NREADS;
+  constexpr int NREAD = MT + NREAD_B;                  // LDS reads per k-step
   constexpr int NMFMA = 4 * MT * Math::SUBSTEPS;       // MFMAs per k-step
   constexpr int READS_PER_SLOT = (NREAD + NMFMA - 1) / NMFMA;
   constexpr int DMA_PER_SLOT = (DMA_B + DMA_A + NMFMA - 1) / NMFMA;
   struct Frags {
-    u32x4 a[MT];
-    typename BT::piece_t b[BT::NREADS];
+    u32x4 a[BPAIR ? MT + 4 : MT];
+    typename BT::piece_t b[BPAIR ? 1 : BT::NREADS];
   };
   // LDS read r of k-step kk of the stage in ring slot `slot`: first the A fragments, then B.
   // `par` = parity of the stage: which half of the pair's 128-byte rows.
@@ -493,11 +497,11 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
     if (r < MT)
       f.a[r] = *reinterpret_cast<const u32x4*>(
           lds + B_RING + pslot * APAIR_BYTES + pair_off(a_frag_row + 32 * r, 4 * par + 2 * kk + g));
-    else if constexpr (BPAIR)
-      f.b[r - MT] = BT::frag_half_pair(lds + slot * BPAIR_BYTES, wn, (r - MT) >> 1, par, kk,
-                                       (r - MT) & 1, l);
-    else
+    else if constexpr (BPAIR) {
+      f.a[r] = BT::frag_pair(lds + slot * BPAIR_BYTES, wn, r - MT, par, kk, l);
+    } else {
       f.b[r - MT] = read_b_piece<BMODE>(lds + slot * OPERAND_BYTES, wn, r - MT, kk, l);
+    }
   };
 
   acc_t acc[MT][4];
@@ -512,7 +516,10 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   // MT need all A fragments (the first reads) but only the first pieces of B.
   auto mfma_piece = [&](const Frags& f, int m) {
     const int sub = m / (4 * MT), j = (m % (4 * MT)) / MT, i = m % MT;
-    acc[i][j] = Math::mfma(BT::bfrag(f.b, j, sub), Math::afrag(f.a[i], sub), acc[i][j]);
+    if constexpr (BPAIR)
+      acc[i][j] = Math::mfma(f.a[MT + j], Math::afrag(f.a[i], sub), acc[i][j]);
+    else
+      acc[i][j] = Math::mfma(BT::bfrag(f.b, j, sub), Math::afrag(f.a[i], sub), acc[i][j]);
   };
 
   Frags f0, f1;
