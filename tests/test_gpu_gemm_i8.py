@@ -119,3 +119,30 @@ def test_quantize_then_gemm_device_pipeline(handle, torch_gpu, oracle, rng):
     # and the quantized product approximates the fp32 product
     ref = X.astype(np.float64) @ W.astype(np.float64).T
     assert np.abs(out.cpu().numpy() - ref).max() < 0.05 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("b_nk", [False, True])
+def test_config_int8_8192(handle, torch_gpu, oracle, b_nk):
+    """int8 8192^3 (the headline size), uniform [-127, 127] from seed 1.  The whole result is
+    pinned by exact integer identities that touch every element -- Freivalds projections
+    C.x = A.(B.x) in int64 and the checksum of checksums sum(C) = colsum(A) . rowsum(B) --
+    and a stratified sample of full rows and columns equals the oracle bit for bit."""
+    n = 8192
+    A, B, _, _ = wl.int8_uniform(n, n, n, seed=1)
+    Bs = np.ascontiguousarray(B.T) if b_nk else B           # stored operand
+    C = handle.gemm_i8_i32(dev(torch_gpu, A), dev(torch_gpu, Bs), ci.B_NK if b_nk else ci.B_KN)
+    assert "mfma" in handle.last_kernel and handle.last_plan == (256, 1)
+    C = C.cpu().numpy()
+    A64, B64, C64 = A.astype(np.int64), B.astype(np.int64), C.astype(np.int64)
+    r = np.random.Generator(np.random.PCG64(11))
+    for _ in range(4):
+        x = r.integers(-3, 4, size=n).astype(np.int64)
+        np.testing.assert_array_equal(C64 @ x, A64 @ (B64 @ x))
+        y = r.integers(-3, 4, size=n).astype(np.int64)
+        np.testing.assert_array_equal(y @ C64, (y @ A64) @ B64)
+    assert int(C.sum(dtype=np.int64)) == int(A64.sum(axis=0) @ B64.sum(axis=1))
+    rows = np.array([0, 1, 31, 32, 255, 256, 257, 4095, 4096, 8190, 8191])
+    np.testing.assert_array_equal(C[rows], oracle.gemm_i8_i32(np.ascontiguousarray(A[rows]), B, False))
+    cols = np.array([0, 3, 4, 127, 128, 255, 256, 4097, 8191])
+    np.testing.assert_array_equal(C[:, cols],
+                                  oracle.gemm_i8_i32(A, np.ascontiguousarray(B[:, cols]), False))
