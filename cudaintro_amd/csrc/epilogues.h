@@ -162,6 +162,7 @@ struct EpiDequantX4 {
   int32_t* acc_out;
   int64_t ldacc;
   static constexpr int OUT_BYTES = OUT_BF16 ? 2 : 4;
+  static constexpr bool REGISTER_HEAVY = DUMP_ACC;  // 256-row tile: stay on the four-wave form
   typedef typename std::conditional<OUT_BF16, u32x2, u32x4>::type packed_t;
   typedef float row_t;   // scale of the row
   typedef f32x4 col_t;   // scales of the four columns

@@ -1,6 +1,8 @@
 // The LDS-tiled MFMA GEMM kernel shared by the bf16, fp16 and int8 families.
 //
-// Workgroup = 256 lanes = 4 waves (2 x 2); macro tile 256 (m) x 256 (n); k is consumed in
+// Workgroup = 256 lanes = 4 waves (2 x 2) -- or, for the 256-row tile of the 16-bit and int8
+// types, 512 lanes = 8 waves (4 x 2) of half the height, two per SIMD, same data flow, see
+// launch_tile_256 --; macro tile 256 (m) x 256 (n); k is consumed in
 // stages of 64 BYTES per row (32 halves, 64 int8 or 16 floats) = two MFMA k-steps.  Each wave
 // owns a 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulators per lane (the AGPR
 // file); one wave per SIMD.  The tile height is a template parameter (MT = 4, 3, 2 or 1 row
@@ -225,6 +227,7 @@ __device__ __forceinline__ typename BTile<MODE>::piece_t read_b_piece(const char
 
 // ---- arithmetic traits ----------------------------------------------------------------------
 struct MathBF16 {
+  static constexpr bool TWO_WAVES_PER_SIMD = true;  // form of the 256-row tile
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
   static constexpr double STAGE_UNIT_US = 0.195;  // one 64 x 256 step of one 64-byte stage
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
@@ -238,6 +241,7 @@ struct MathBF16 {
   }
 };
 struct MathF16 {
+  static constexpr bool TWO_WAVES_PER_SIMD = true;
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
   static constexpr double STAGE_UNIT_US = 0.195;
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
@@ -250,6 +254,7 @@ struct MathF16 {
   }
 };
 struct MathI8 {
+  static constexpr bool TWO_WAVES_PER_SIMD = true;
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
   static constexpr double STAGE_UNIT_US = 0.195;
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
@@ -266,6 +271,7 @@ struct MathI8 {
 // A 16-byte fragment read gives a lane 4 consecutive k of its row, lanes 32-63 the next 4,
 // so four MFMAs consume one fragment pair: MFMA e multiplies k0+e (lanes 0-31) and k0+4+e.
 struct MathF32 {
+  static constexpr bool TWO_WAVES_PER_SIMD = false;
   static constexpr int SUBSTEPS = 4;
   static constexpr double STAGE_UNIT_US = 0.95;
   static __device__ __forceinline__ float afrag(u32x4 a, int sub) {
@@ -343,8 +349,8 @@ __device__ __forceinline__ EpiPartialX4 epilogue_of_split(const EpiPartialX4& e,
 // A, B are byte pointers; lda/ldb are in BYTES.  Any M; N a multiple of 4; all rows 16-byte
 // aligned (tile_shape_ok checks).  KTS = number of 64-byte stages of this workgroup's K
 // range; grid = (tiles, K ranges).
-template <typename Math, int BMODE, int NSTAGES, int MT, typename Epi>
-__global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int tiles_m,
+template <typename Math, int BMODE, int NSTAGES, int MT, typename Epi, int WM = 2>
+__global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, int tiles_m,
                                                            int tiles_n, int KTS,
                                                            const char* __restrict__ A,
                                                            int64_t lda,
@@ -360,18 +366,19 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   typedef typename Math::acc_t acc_t;
   typedef BTile<BMODE> BT;
   constexpr int DIST = NSTAGES - 1;  // stages in flight ahead of the one being multiplied
-  constexpr int TILE_M = 64 * MT;    // rows of the macro tile
+  constexpr int NW = 2 * WM;             // waves: WM rows of 2
+  constexpr int TILE_M = 32 * MT * WM;   // rows of the macro tile
   static_assert(NSTAGES == 4, "the wait counts below assume three stages in flight");
   // N x K weights are row-major like A: they too are fetched as whole 128-byte lines, a pair
   // of stages at a time, into two 32 KiB pair slots (the same 64 KiB as the ring of four
   // single stages the K x N layouts use).
   constexpr bool BPAIR = BMODE == B_NK;
-  constexpr int DMA_A = 2 * MT;          // per wave and stage pair: A instructions of 1 KiB
-  constexpr int DMA_B = BPAIR ? 8 : 4;   // per wave: B instructions per stage pair / per stage
+  constexpr int DMA_A = TILE_M / 8 / NW;        // per wave and stage pair: A instructions of 1 KiB
+  constexpr int DMA_B = (BPAIR ? 32 : 16) / NW; // per wave: B instructions per stage pair / per stage
   constexpr int BPAIR_BYTES = 256 * 128;
   constexpr int APAIR_BYTES = TILE_M * 128;
   constexpr int B_RING = NSTAGES * OPERAND_BYTES;   // B slots first, then three A pair slots
-  typedef RowPairDmaT<MT> ADma;
+  typedef RowPairDmaT<1> PairDma;   // instruction q = rows 8 q .. 8 q + 7: (q >> 1, q & 1)
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int t = threadIdx.x;
   const int l = t & 63;
@@ -410,7 +417,7 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   uint32_t a_hi = 0;
 #pragma unroll
   for (int i = 0; i < DMA_A; ++i) {
-    const int r = 16 * MT * w + 8 * i + (l >> 3);
+    const int r = 8 * (DMA_A * w + i) + (l >> 3);
     a_hi |= (uint32_t)((((l & 7) ^ pair_swz(r)) >> 2) & 1) << i;
   }
   const int last_pair = (KTS - 1) >> 1;
@@ -418,18 +425,23 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   uint32_t b_hi = 0;  // the same for the rows of N x K weights
   if (BPAIR) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int r = 64 * w + 8 * i + (l >> 3);
+    for (int i = 0; i < DMA_B; ++i) {
+      const int r = 8 * (DMA_B * w + i) + (l >> 3);
       b_hi |= (uint32_t)((((l & 7) ^ pair_swz(r)) >> 2) & 1) << i;
     }
   }
   uint32_t a_voff[DMA_A], b_voff[DMA_B];
 #pragma unroll
-  for (int i = 0; i < DMA_A; ++i) a_voff[i] = (uint32_t)ADma::dma_src(w, i, l, lda, a_last);
+  for (int i = 0; i < DMA_A; ++i) {
+    const int q = DMA_A * w + i;
+    a_voff[i] = (uint32_t)PairDma::dma_src(q >> 1, q & 1, l, lda, a_last);
+  }
 #pragma unroll
-  for (int i = 0; i < DMA_B; ++i)
-    b_voff[i] = BPAIR ? (uint32_t)RowPairDmaT<4>::dma_src(w, i, l, ldb, b_last)
-                      : (uint32_t)BT::dma_src(w, i, l, ldb, b_last);
+  for (int i = 0; i < DMA_B; ++i) {
+    const int q = DMA_B * w + i;
+    b_voff[i] = BPAIR ? (uint32_t)PairDma::dma_src(q >> 1, q & 1, l, ldb, b_last)
+                      : (uint32_t)BT::dma_src(q >> 2, q & 3, l, ldb, b_last);
+  }
 
   // The DMA instructions are written as asm so that the compiler's wait-count insertion does
   // not know them: it would otherwise make every later LDS read it cannot tell apart (the
@@ -462,16 +474,17 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
         uint32_t off = b_voff[d];
         if (tail_pair) off -= ((b_hi >> d) & 1u) << 6;
         dma16(b_tile + (int64_t)(st >> 1) * 128, off,
-              lds_base + slot * BPAIR_BYTES + RowPairDmaT<4>::dma_lds(w, d));
+              lds_base + slot * BPAIR_BYTES + PairDma::dma_lds((DMA_B * w + d) >> 1, (DMA_B * w + d) & 1));
       } else {
         dma16(b_tile + (int64_t)st * b_kstep, b_voff[d],
-              lds_base + slot * OPERAND_BYTES + BT::dma_lds(w, d));
+              lds_base + slot * OPERAND_BYTES + BT::dma_lds((DMA_B * w + d) >> 2, (DMA_B * w + d) & 3));
       }
     } else {
       uint32_t off = a_voff[d - DMA_B];
       if (tail_pair) off -= ((a_hi >> (d - DMA_B)) & 1u) << 6;
       dma16(a_tile + (int64_t)(st >> 1) * 128, off,
-            lds_base + B_RING + pslot * APAIR_BYTES + ADma::dma_lds(w, d - DMA_B));
+            lds_base + B_RING + pslot * APAIR_BYTES +
+                PairDma::dma_lds((DMA_A * w + d - DMA_B) >> 1, (DMA_A * w + d - DMA_B) & 1));
     }
   };
   typedef std::integral_constant<bool, true> steady_t;
@@ -636,6 +649,8 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
   constexpr int ROW_STRIDE = ROW_BYTES + 16;
   constexpr int LANES_PER_ROW = ROW_BYTES / 16;
   constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+  static_assert(NW * 32 * ROW_STRIDE <= NSTAGES * OPERAND_BYTES + 3 * APAIR_BYTES,
+                "the waves' staging blocks must fit the ring");
   char* scr = lds + w * (32 * ROW_STRIDE);
   typedef decltype(epi.pack((int64_t)0, (int64_t)0, acc[0][0][0], acc[0][0][0], acc[0][0][0],
                             acc[0][0][0])) packed_t;
@@ -686,26 +701,27 @@ __global__ __launch_bounds__(256, 1) void mfma_tile_kernel(int M, int N, int til
 
 constexpr int DEFAULT_STAGES = 4;
 
-template <typename Math, int BMODE, int MT, typename Epi>
+template <typename Math, int BMODE, int MT, typename Epi, int WM = 2>
 void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
                     int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi,
                     int splits = 1) {
   constexpr int NSTAGES = DEFAULT_STAGES;
-  constexpr int LDS_BYTES = NSTAGES * OPERAND_BYTES + 3 * (64 * MT * 128);
-  auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, MT, Epi>;
+  constexpr int TILE_M = 32 * MT * WM;
+  constexpr int LDS_BYTES = NSTAGES * OPERAND_BYTES + 3 * (TILE_M * 128);
+  auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, MT, Epi, WM>;
   static int attr_device = -1;  // one per template instance
   if (attr_device != ctx->device) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                               LDS_BYTES);
     attr_device = ctx->device;
   }
-  const int tiles_m = (int)((M + 64 * MT - 1) / (64 * MT)), tiles_n = (int)((N + BN - 1) / BN);
-  ctx->last_tile_rows = 64 * MT;
+  const int tiles_m = (int)((M + TILE_M - 1) / TILE_M), tiles_n = (int)((N + BN - 1) / BN);
+  ctx->last_tile_rows = TILE_M;
   ctx->last_k_splits = splits;
   const int64_t kts = K_bytes / KB / splits;  // stages per K range
   const int64_t a_step = kts * KB;
   const int64_t b_step = BMODE == B_NK ? kts * KB : kts * (KB / Math::ELEM_BYTES) * ldb_bytes;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(256),
+  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(128 * WM),
                      LDS_BYTES, ctx->stream, (int)M, (int)N, tiles_m, tiles_n, (int)kts,
                      static_cast<const char*>(A), lda_bytes, static_cast<const char*>(B),
                      ldb_bytes, epi, a_step, b_step);
@@ -811,12 +827,36 @@ inline int best_mt(int64_t M, int64_t N, int cus, double* cost = nullptr) {
   return best;
 }
 
+// An epilogue may declare `static constexpr bool REGISTER_HEAVY = true` to stay on the
+// four-wave form of the 256-row tile (512 registers per wave instead of 256).
+template <typename E, typename = void>
+struct epi_register_heavy : std::false_type {};
+template <typename E>
+struct epi_register_heavy<E, typename std::enable_if<E::REGISTER_HEAVY>::type> : std::true_type {};
+
+// The 256-row tile: eight waves of 64 x 128 (two per SIMD: while one wave issues a DMA the
+// other issues MFMAs) for the 16-bit and int8 types, four waves of 128 x 128 for fp32 (whose
+// MFMA shares the vector ALU: a second wave per SIMD gains nothing) and for register-heavy
+// epilogues.  Both forms fetch, multiply and store the same data in the same order: results
+// are identical bit for bit.
+template <typename Math, int BMODE, typename Epi>
+void launch_tile_256(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
+                     int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi,
+                     int splits = 1) {
+  if constexpr (Math::TWO_WAVES_PER_SIMD && !epi_register_heavy<Epi>::value)
+    launch_tile_mt<Math, BMODE, 2, Epi, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi,
+                                           splits);
+  else
+    launch_tile_mt<Math, BMODE, 4, Epi, 2>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi,
+                                           splits);
+}
+
 template <typename Math, int BMODE, typename Epi>
 void launch_tile_any_mt(cigemmContext* ctx, int mt, int64_t M, int64_t N, int64_t K_bytes,
                         const void* A, int64_t lda_bytes, const void* B, int64_t ldb_bytes,
                         const Epi& epi, int splits = 1) {
   if (mt == 4)
-    launch_tile_mt<Math, BMODE, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
+    launch_tile_256<Math, BMODE>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
   else if (mt == 3)
     launch_tile_mt<Math, BMODE, 3>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
   else if (mt == 2)
@@ -868,7 +908,7 @@ bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
         double rest = 0;
         const int mt2 = best_mt(M, n2, cus, &rest);
         if (tile_plan_cost(M, n1, 4, cus) + rest < single * 0.97) {
-          launch_tile_mt<Math, BMODE, 4>(ctx, M, n1, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+          launch_tile_256<Math, BMODE>(ctx, M, n1, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
           const char* B2 = static_cast<const char*>(B) +
                            (BMODE == B_NK ? n1 * ldb_bytes : n1 * Math::ELEM_BYTES);
           launch_tile_any_mt<Math, BMODE>(ctx, mt2, M, n2, K_bytes, A, lda_bytes, B2, ldb_bytes,
