@@ -1,7 +1,7 @@
 // The LDS-tiled MFMA GEMM kernel shared by the bf16, fp16 and int8 families.
 //
-// Workgroup = 256 lanes = 4 waves (2 x 2) -- or, for the 256-row tile of the 16-bit and int8
-// types, 512 lanes = 8 waves (4 x 2) of half the height, two per SIMD, same data flow, see
+// Workgroup = 256 lanes = 4 waves (2 x 2) -- or, for the 256-row tile over N x K int8 weights,
+// 512 lanes = 8 waves (4 x 2) of half the height, two per SIMD, same data flow, see
 // launch_tile_256 --; macro tile 256 (m) x 256 (n); k is consumed in
 // stages of 64 BYTES per row (32 halves, 64 int8 or 16 floats) = two MFMA k-steps.  Each wave
 // owns a 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulators per lane (the AGPR
@@ -227,7 +227,6 @@ __device__ __forceinline__ typename BTile<MODE>::piece_t read_b_piece(const char
 
 // ---- arithmetic traits ----------------------------------------------------------------------
 struct MathBF16 {
-  static constexpr bool TWO_WAVES_PER_SIMD = true;  // form of the 256-row tile
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
   static constexpr double STAGE_UNIT_US = 0.195;  // one 64 x 256 step of one 64-byte stage
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
@@ -241,7 +240,6 @@ struct MathBF16 {
   }
 };
 struct MathF16 {
-  static constexpr bool TWO_WAVES_PER_SIMD = true;
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
   static constexpr double STAGE_UNIT_US = 0.195;
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
@@ -254,7 +252,6 @@ struct MathF16 {
   }
 };
 struct MathI8 {
-  static constexpr bool TWO_WAVES_PER_SIMD = true;
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
   static constexpr double STAGE_UNIT_US = 0.195;
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
@@ -271,7 +268,6 @@ struct MathI8 {
 // A 16-byte fragment read gives a lane 4 consecutive k of its row, lanes 32-63 the next 4,
 // so four MFMAs consume one fragment pair: MFMA e multiplies k0+e (lanes 0-31) and k0+4+e.
 struct MathF32 {
-  static constexpr bool TWO_WAVES_PER_SIMD = false;
   static constexpr int SUBSTEPS = 4;
   static constexpr double STAGE_UNIT_US = 0.95;
   static __device__ __forceinline__ float afrag(u32x4 a, int sub) {
@@ -834,16 +830,19 @@ struct epi_register_heavy : std::false_type {};
 template <typename E>
 struct epi_register_heavy<E, typename std::enable_if<E::REGISTER_HEAVY>::type> : std::true_type {};
 
-// The 256-row tile: eight waves of 64 x 128 (two per SIMD: while one wave issues a DMA the
-// other issues MFMAs) for the 16-bit and int8 types, four waves of 128 x 128 for fp32 (whose
-// MFMA shares the vector ALU: a second wave per SIMD gains nothing) and for register-heavy
-// epilogues.  Both forms fetch, multiply and store the same data in the same order: results
-// are identical bit for bit.
+// The 256-row tile has two forms that fetch, multiply and store the same data in the same
+// order (results identical bit for bit): four waves of 128 x 128, one per SIMD, and eight waves
+// of 64 x 128, two per SIMD, where one wave's DMA issue hides under the other's MFMAs at 1.5 x
+// the LDS fragment traffic.  The second takes 7 % fewer cycles, but in sustained runs the
+// chip is power limited and answers with a lower clock: bf16 on N(0,1) data -0.5 % in time,
+// int8 K x N +-0.4 %, int8 N x K +1.4..2.1 % (200 launches each, alternating, one box; +1..4 %
+// everywhere in short runs on low-entropy data), fp32 +0.2 % (its MFMA shares the vector ALU).
+// So only N x K int8 weights use it.
 template <typename Math, int BMODE, typename Epi>
 void launch_tile_256(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
                      int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi,
                      int splits = 1) {
-  if constexpr (Math::TWO_WAVES_PER_SIMD && !epi_register_heavy<Epi>::value)
+  if constexpr (BMODE == B_NK && !epi_register_heavy<Epi>::value)
     launch_tile_mt<Math, BMODE, 2, Epi, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi,
                                            splits);
   else
