@@ -67,6 +67,36 @@ def median_call_ms(torch, fn, steps):
     return float(np.median([a.elapsed_time(b) for a, b in evs]))
 
 
+def graph_call_us(torch, ci, make_call, calls=24, replays=10):
+    """Per-call time of `calls` library calls recorded once into a HIP graph on a side stream
+    (with a handle of its own bound to that stream) and replayed: what a serving loop that
+    captures its decode step sees, without per-launch host work.  make_call(handle, i) issues
+    call number i."""
+    side = torch.cuda.Stream()
+    h = ci.Handle(stream=side)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for i in range(calls):
+            make_call(h, i)                      # eager once: loads code objects
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for i in range(calls):
+            make_call(h, i)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    h.close()
+    return e0.elapsed_time(e1) * 1e3 / (replays * calls)
+
+
 def dev16(torch, bits, kind):
     if kind == "bf16":
         return torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
@@ -266,6 +296,9 @@ def main():
             per_config[f"skinny_bf16_M{M}"] = {"gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS,
                                                "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
                                                "bytes": nbytes, "kernel": handle.last_kernel}
+            if M == 1:
+                per_config["skinny_bf16_M1"]["us_replayed_from_graph"] = graph_call_us(
+                    torch, ci, lambda hh, i: hh.gemm_bf16(x, ws[i & 3], out=y))
             del ws
             xq, sx, wq, sw = wl.skinny_int8(M, 8192, 8192, seed=4)
             xd, sxd, swd = torch.from_numpy(xq).cuda(), torch.from_numpy(sx).cuda(), torch.from_numpy(sw).cuda()
@@ -281,6 +314,10 @@ def main():
             per_config[f"skinny_int8_M{M}"] = {"gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS,
                                                "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
                                                "bytes": nbytes, "kernel": handle.last_kernel}
+            if M == 1:
+                per_config["skinny_int8_M1"]["us_replayed_from_graph"] = graph_call_us(
+                    torch, ci, lambda hh, i: hh.gemm_i8_dequant(xd, wqs[i % 6], sxd, swd, ci.B_NK,
+                                                                ci.OUT_BF16, out=yo))
             del wqs
         # small-batch shapes between the decode and the square configurations: few output
         # tiles and a long K, run as split-K (weights still dominate the traffic)
