@@ -42,7 +42,7 @@ def test_fill_i8(oracle):
         assert a.min() == -127 and a.max() == 127
 
 
-def test_survey_known_answers(oracle):
+def test_hand_checked_known_answers(oracle):
     """Hand-checked decimal values for the first elements of the 4096^2 operands."""
     a = oracle.fill_random_f32(1 << 24, 0x3234)
     np.testing.assert_array_equal(
