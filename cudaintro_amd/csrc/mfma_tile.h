@@ -37,13 +37,14 @@
 // Pipeline, iteration s (B of stage s sits in slot s % 4, A in pair slot (s / 2) % 3):
 //   k-step 0: 16 MFMAs on the fragments of (s,0); under them the 12 LDS reads of (s,1)
 //   wait until this wave's DMA of stage s+1 has landed (vmcnt), workgroup barrier
-//   k-step 1: 16 MFMAs on (s,1); under them the 12 LDS reads of (s+1,0) and the DMA of
-//             stage s+3: 4 instructions of B into the slot stage s-1 just left (every wave
-//             finished reading it before it reached the barrier) and, for odd s, the 8 of
-//             the A pair of stages s+3 and s+4.
-// With N x K weights both operands move as pairs: odd stages issue the B pair and the A pair
-// of stages s+3, s+4 (16 instructions, the B pair into the slot whose last fragments were
-// read in k-step 0 of this stage), even stages none.
+//   k-step 1: 16 MFMAs on (s,1); under them the 12 LDS reads of (s+1,0) and the DMA:
+//             4 instructions of B of stage s+3 into the slot stage s-1 just left (every wave
+//             finished reading it before it reached the barrier) and 4 of the 8 of an A
+//             pair: the first half of the pair of stages s+4, s+5 when s is even, the second
+//             half of the same pair (then stages s+3, s+4) when s is odd.
+// With N x K weights both operands move as pairs: even stages issue the A pair of stages s+4,
+// s+5, odd stages the B pair of stages s+3, s+4 (into the slot whose last fragments were read
+// in k-step 0 of that stage).
 // Fragments are double buffered in registers.  The emitted order is pinned slot by slot
 // with scheduling fences: one MFMA, at most one LDS read, at most one DMA.
 //
@@ -495,7 +496,9 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   constexpr int NREAD = MT + NREAD_B;                  // LDS reads per k-step
   constexpr int NMFMA = 4 * MT * Math::SUBSTEPS;       // MFMAs per k-step
   constexpr int READS_PER_SLOT = (NREAD + NMFMA - 1) / NMFMA;
-  constexpr int DMA_PER_SLOT = (DMA_B + DMA_A + NMFMA - 1) / NMFMA;
+  static_assert(DMA_A % 2 == 0, "an A pair is issued in two halves");
+  constexpr int DMA_PER_SLOT =
+      ((BPAIR ? (DMA_A > DMA_B ? DMA_A : DMA_B) : DMA_B + DMA_A / 2) + NMFMA - 1) / NMFMA;
   struct Frags {
     u32x4 a[BPAIR ? MT + 4 : MT];
     typename BT::piece_t b[BPAIR ? 1 : BT::NREADS];
@@ -562,12 +565,15 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   // advance every second stage.
   int slot = 0, next_slot = 1, dma_slot = DIST;
   int pslot = 0, next_pslot = 1, dma_pslot = 2;
-  // One stage; PAR = its parity.  Single B stages: even stages issue B[s+3] only, odd stages
-  // B[s+3] and the A pair of stages s+3, s+4.  B pairs: odd stages issue both pairs of stages
-  // s+3, s+4, even stages nothing.
+  // One stage; PAR = its parity.  Single B stages: every stage issues B[s+3] and half of an A
+  // pair: an even stage the first half of the pair of stages s+4, s+5 (its slot, one of three,
+  // has been free since the stage before), the odd stage after it the second half.  B pairs: even stages issue the A pair of stages
+  // s+4, s+5 (its slot, one of three, has been free since the stage before), odd stages the B
+  // pair of stages s+3, s+4 (its slot, one of two, is the one this stage stops reading): the
+  // instructions of a stage pair are spread over both of its stages.
   auto stage = [&](int s, auto par_const, auto steady_const) {
     constexpr int PAR = decltype(par_const)::value;
-    constexpr int NDMA = BPAIR ? (PAR ? DMA_B + DMA_A : 0) : (PAR ? DMA_B + DMA_A : DMA_B);
+    constexpr int NDMA = BPAIR ? (PAR ? DMA_B : DMA_A) : DMA_B + DMA_A / 2;
 #pragma unroll
     for (int sl = 0; sl < NMFMA; ++sl) {
       mfma_piece(f0, sl);
@@ -577,17 +583,19 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
       __builtin_amdgcn_sched_barrier(0);
     }
     if (BPAIR) {
-      // Odd stage: the next pair (issued two stages ago, nothing newer in flight) landed;
-      // this wave's last reads of the current B pair slot are complete before any wave
-      // refills it after the barrier.  Even stage: stage s+1 is in the pair already landed.
+      // Odd stage: the next pair of both operands landed (only the A pair issued one stage ago
+      // may still be in flight); this wave's last reads of the current B pair slot are
+      // complete before any wave refills it after the barrier.  Even stage: stage s+1 is in
+      // the pair already landed.
       if (PAR) {
-        wait_vmcnt(std::integral_constant<int, 0>{});
+        wait_vmcnt(std::integral_constant<int, DMA_A>{});
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }
     } else {
       // stage s+1 landed for this wave.  Still in flight, in issue order after what stage
-      // s+1 needs: even s: B[s+2] and the A pair (s+2, s+3); odd s: B[s+2].
-      wait_vmcnt(std::integral_constant<int, PAR ? DMA_B : DMA_B + DMA_A>{});
+      // s+1 needs: even s: the first half of the A pair (s+2, s+3), B[s+2] and its second
+      // half; odd s: B[s+2] and the first half of the A pair (s+3, s+4).
+      wait_vmcnt(std::integral_constant<int, PAR ? DMA_B + DMA_A / 2 : DMA_B + DMA_A>{});
     }
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -601,7 +609,21 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
                      PAR ^ 1, 0, r);
 #pragma unroll
       for (int d = sl * DMA_PER_SLOT; d < (sl + 1) * DMA_PER_SLOT; ++d)
-        if (d < NDMA) dma_piece(s + DIST, BPAIR ? slot : dma_slot, dma_pslot, d, steady_const);
+        if (d < NDMA) {
+          if (BPAIR) {
+            if (PAR)
+              dma_piece(s + DIST, slot, dma_pslot, d, steady_const);               // B pair
+            else
+              dma_piece(s + DIST + 1, slot, dma_pslot, DMA_B + d, steady_const);   // A pair
+          } else if (d < DMA_B) {
+            dma_piece(s + DIST, dma_slot, dma_pslot, d, steady_const);             // B[s+3]
+          } else {
+            // half of the A pair the DMA is filling: stages s+4, s+5 seen from an even stage,
+            // s+3, s+4 from the odd stage after it
+            dma_piece(PAR ? s + DIST : s + DIST + 1, dma_slot, dma_pslot,
+                      d + (PAR ? DMA_A / 2 : 0), steady_const);
+          }
+        }
       __builtin_amdgcn_sched_barrier(0);
     }
     if (BPAIR) {
