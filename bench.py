@@ -296,9 +296,6 @@ def main():
             per_config[f"skinny_bf16_M{M}"] = {"gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS,
                                                "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
                                                "bytes": nbytes, "kernel": handle.last_kernel}
-            if M == 1:
-                per_config["skinny_bf16_M1"]["us_replayed_from_graph"] = graph_call_us(
-                    torch, ci, lambda hh, i: hh.gemm_bf16(x, ws[i & 3], out=y))
             del ws
             xq, sx, wq, sw = wl.skinny_int8(M, 8192, 8192, seed=4)
             xd, sxd, swd = torch.from_numpy(xq).cuda(), torch.from_numpy(sx).cuda(), torch.from_numpy(sw).cuda()
@@ -314,10 +311,6 @@ def main():
             per_config[f"skinny_int8_M{M}"] = {"gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS,
                                                "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
                                                "bytes": nbytes, "kernel": handle.last_kernel}
-            if M == 1:
-                per_config["skinny_int8_M1"]["us_replayed_from_graph"] = graph_call_us(
-                    torch, ci, lambda hh, i: hh.gemm_i8_dequant(xd, wqs[i % 6], sxd, swd, ci.B_NK,
-                                                                ci.OUT_BF16, out=yo))
             del wqs
         # small-batch shapes between the decode and the square configurations: few output
         # tiles and a long K, run as split-K (weights still dominate the traffic)
@@ -339,6 +332,25 @@ def main():
                                               "peak": PEAK_HBM_GBS, "us": e / args.steps * 1e6,
                                               "bytes": nbytes, "kernel": handle.last_kernel}
             del ws
+
+        # The decode shape once more, as replays of a captured HIP graph.  Last of the GEMM
+        # measurements on purpose: once a second stream has been used in the process, eager
+        # launches on the first one take a few microseconds longer each.
+        xb, wb = wl.skinny_bf16(1, 8192, 8192, seed=4)
+        x = dev16(torch, xb, "bf16")
+        ws = [dev16(torch, wb, "bf16") for _ in range(4)]
+        y = torch.empty((1, 8192), dtype=torch.bfloat16, device="cuda")
+        per_config["skinny_bf16_M1"]["us_replayed_from_graph"] = graph_call_us(
+            torch, ci, lambda hh, i: hh.gemm_bf16(x, ws[i & 3], out=y))
+        del ws
+        xq, sx, wq, sw = wl.skinny_int8(1, 8192, 8192, seed=4)
+        xd, sxd, swd = torch.from_numpy(xq).cuda(), torch.from_numpy(sx).cuda(), torch.from_numpy(sw).cuda()
+        wqs = [torch.from_numpy(wq).cuda() for _ in range(6)]
+        yo = torch.empty((1, 8192), dtype=torch.bfloat16, device="cuda")
+        per_config["skinny_int8_M1"]["us_replayed_from_graph"] = graph_call_us(
+            torch, ci, lambda hh, i: hh.gemm_i8_dequant(xd, wqs[i % 6], sxd, swd, ci.B_NK,
+                                                        ci.OUT_BF16, out=yo))
+        del wqs
 
         # What the matrix cores sustain with no memory traffic at all, at the clock the chip
         # holds under that load, on constant and on random operand bits.
