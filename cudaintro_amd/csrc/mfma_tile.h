@@ -667,8 +667,8 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   constexpr int ROW_STRIDE = ROW_BYTES + 16;
   constexpr int LANES_PER_ROW = ROW_BYTES / 16;
   constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
-  static_assert(NW * 32 * ROW_STRIDE <= NSTAGES * OPERAND_BYTES + 3 * APAIR_BYTES,
-                "the waves' staging blocks must fit the ring");
+  // (the launcher sizes the dynamic LDS for the larger of the ring and these staging blocks)
+  static_assert(NW * 32 * ROW_STRIDE <= 160 * 1024, "the waves' staging blocks must fit the LDS");
   char* scr = lds + w * (32 * ROW_STRIDE);
   typedef decltype(epi.pack((int64_t)0, (int64_t)0, acc[0][0][0], acc[0][0][0], acc[0][0][0],
                             acc[0][0][0])) packed_t;
@@ -725,7 +725,9 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
                     int splits = 1) {
   constexpr int NSTAGES = DEFAULT_STAGES;
   constexpr int TILE_M = 32 * MT * WM;
-  constexpr int LDS_BYTES = NSTAGES * OPERAND_BYTES + 3 * (TILE_M * 128);
+  constexpr int RING_BYTES = NSTAGES * OPERAND_BYTES + 3 * (TILE_M * 128);
+  constexpr int STAGING_BYTES = 2 * WM * 32 * (128 * Epi::OUT_BYTES + 16);   // epilogue, per wave
+  constexpr int LDS_BYTES = RING_BYTES > STAGING_BYTES ? RING_BYTES : STAGING_BYTES;
   auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, MT, Epi, WM>;
   static int attr_device = -1;  // one per template instance
   if (attr_device != ctx->device) {
@@ -872,6 +874,21 @@ void launch_tile_256(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, 
                                            splits);
 }
 
+// The 128-row tile has the same two forms (four waves of 64 x 128, eight of 32 x 128); with
+// N x K int8 weights the second is 9 % faster (2048 x 11008 x 4096: 108 -> 98 us), with K x N
+// operands 2 % slower (their transposing fragment reads are twice as many instructions).
+template <typename Math, int BMODE, typename Epi>
+void launch_tile_128(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
+                     int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi,
+                     int splits = 1) {
+  if constexpr (BMODE == B_NK && !epi_register_heavy<Epi>::value)
+    launch_tile_mt<Math, BMODE, 1, Epi, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi,
+                                           splits);
+  else
+    launch_tile_mt<Math, BMODE, 2, Epi, 2>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi,
+                                           splits);
+}
+
 template <typename Math, int BMODE, typename Epi>
 void launch_tile_any_mt(cigemmContext* ctx, int mt, int64_t M, int64_t N, int64_t K_bytes,
                         const void* A, int64_t lda_bytes, const void* B, int64_t ldb_bytes,
@@ -881,7 +898,7 @@ void launch_tile_any_mt(cigemmContext* ctx, int mt, int64_t M, int64_t N, int64_
   else if (mt == 3)
     launch_tile_mt<Math, BMODE, 3>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
   else if (mt == 2)
-    launch_tile_mt<Math, BMODE, 2>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
+    launch_tile_128<Math, BMODE>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
   else
     launch_tile_mt<Math, BMODE, 1>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
 }
