@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X quantization-GEMM library.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu] [--reference-seconds S]
 
 Headline (the one JSON line printed last): bf16 GEMM 8192^3, TFLOP/s = 2*M*N*K / time, inputs
 resident in HBM before the timed region; one "step" is one GEMM call.  The same line carries
@@ -97,6 +97,27 @@ def graph_call_us(torch, ci, make_call, calls=24, replays=10):
     return e0.elapsed_time(e1) * 1e3 / (replays * calls)
 
 
+def reference_protocol(seconds):
+    """The reference's own measurement (quantization/main.cu:8-31, GEMM_*.cu:59-84): the suite
+    driver built beside the library, as a child process: 4096^3 per precision, device-side
+    fills with the reference's seeds, one warm-up, a wall-clock loop of at least `seconds`
+    sampled every 256 launches.  Returns {"BF16": TFLOP/s, ...} or None if it is not built."""
+    import re
+    import subprocess
+    exe = os.path.join(ROOT, "cudaintro_amd", "gemm_suite")
+    if not os.path.exists(exe):
+        return None
+    out = subprocess.run([exe, "--seconds", str(seconds)], capture_output=True, text=True,
+                         timeout=60 + 8 * seconds)
+    if out.returncode != 0:
+        log("[bench] gemm_suite failed: " + out.stderr.strip()[-300:])
+        return None
+    res = {"seconds_per_precision": seconds, "size": 4096}
+    for m in re.finditer(r"Ran (\d+) (\w+) GEMMs in ([\d.]+) s \(([\d.]+) TFLOP/s\)", out.stdout):
+        res[m.group(2)] = float(m.group(4))
+    return res
+
+
 def dev16(torch, bits, kind):
     if kind == "bf16":
         return torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
@@ -144,6 +165,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--reference-seconds", type=float, default=3.0,
+                    help="time budget per precision of the reference's own protocol (its driver "
+                         "uses 10; 0 skips that leg)")
     ap.add_argument("--size", type=int, default=8192, help="headline M=N=K (default 8192)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy a few times (reference point for "
@@ -351,6 +375,13 @@ def main():
             torch, ci, lambda hh, i: hh.gemm_i8_dequant(xd, wqs[i % 6], sxd, swd, ci.B_NK,
                                                         ci.OUT_BF16, out=yo))
         del wqs
+
+        if args.reference_seconds > 0:
+            log("[bench] the reference's protocol (gemm_suite, 4096^3) ...")
+            torch.cuda.synchronize()
+            ref = reference_protocol(args.reference_seconds)
+            if ref:
+                per_config["reference_protocol_4096"] = ref
 
         # What the matrix cores sustain with no memory traffic at all, at the clock the chip
         # holds under that load, on constant and on random operand bits.
