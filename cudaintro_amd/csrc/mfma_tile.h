@@ -1,8 +1,8 @@
 // The LDS-tiled MFMA GEMM kernel shared by the bf16, fp16 and int8 families.
 //
-// Workgroup = 256 lanes = 4 waves (2 x 2) -- or, for the 256-row tile over N x K int8 weights,
-// 512 lanes = 8 waves (4 x 2) of half the height, two per SIMD, same data flow, see
-// launch_tile_256 --; macro tile 256 (m) x 256 (n); k is consumed in
+// Workgroup = 256 lanes = 4 waves (2 x 2) -- or, for the 256- and 128-row tiles over N x K int8
+// weights, 512 lanes = 8 waves (4 x 2) of half the height, two per SIMD, same data flow, see
+// launch_tile_256 / launch_tile_128 --; macro tile 256 (m) x 256 (n); k is consumed in
 // stages of 64 BYTES per row (32 halves, 64 int8 or 16 floats) = two MFMA k-steps.  Each wave
 // owns a 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulators per lane (the AGPR
 // file); one wave per SIMD.  The tile height is a template parameter (MT = 4, 3, 2 or 1 row
