@@ -861,17 +861,28 @@ struct epi_register_heavy<E, typename std::enable_if<E::REGISTER_HEAVY>::type> :
 // chip is power limited and answers with a lower clock: bf16 on N(0,1) data -0.5 % in time,
 // int8 K x N +-0.4 %, int8 N x K +1.4..2.1 % (200 launches each, alternating, one box; +1..4 %
 // everywhere in short runs on low-entropy data), fp32 +0.2 % (its MFMA shares the vector ALU).
-// So only N x K int8 weights use it.
+// With one round of tiles (4096^3: 256 tiles, 1000 launches on N(0,1) data) bf16 gains 1.9 %,
+// int8 K x N loses 2 %.  So N x K int8 weights use it always, the 16-bit types when the tiles
+// fit one round.
 template <typename Math, int BMODE, typename Epi>
 void launch_tile_256(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
                      int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi,
                      int splits = 1) {
-  if constexpr (BMODE == B_NK && !epi_register_heavy<Epi>::value)
+  if constexpr (BMODE == B_NK && !epi_register_heavy<Epi>::value) {
     launch_tile_mt<Math, BMODE, 2, Epi, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi,
                                            splits);
-  else
+  } else {
+    if constexpr (Math::ELEM_BYTES == 2 && !epi_register_heavy<Epi>::value) {
+      const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+      if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) * splits <= cus) {
+        launch_tile_mt<Math, BMODE, 2, Epi, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes,
+                                               epi, splits);
+        return;
+      }
+    }
     launch_tile_mt<Math, BMODE, 4, Epi, 2>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi,
                                            splits);
+  }
 }
 
 // The 128-row tile has the same two forms (four waves of 64 x 128, eight of 32 x 128); with
