@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 # (M, N) -> expected tile rows on 256 CUs: the height whose tiles just fill one round
 HEIGHTS = [((4096, 4096), 256), ((3072, 4096), 192), ((2048, 4096), 128), ((1024, 4096), 64),
-           ((3000, 4096), 192), ((1999, 4080), 128)]
+           ((3000, 4096), 192), ((1999, 4080), 128), ((4000, 4080), 256), ((1000, 4080), 64)]
 
 
 def _skip_unless_256_cus(torch):
