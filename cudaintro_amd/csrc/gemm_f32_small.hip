@@ -1,8 +1,15 @@
 // fp32 GEMM for problems too small (or too narrow) to fill the chip with 256-column tiles:
 // one 32x32 output tile per 256-lane workgroup, the k range split over the four waves
-// (each wave: v_mfma_f32_32x32x2_f32 on operands loaded straight from global memory into
-// registers, no LDS staging), the four partial tiles summed through LDS in wave order
-// (deterministic), then bias / activation and the store.  512^3 gives 256 workgroups
+// (each wave: v_mfma_f32_32x32x2_f32 on operands loaded straight from global memory, no
+// workgroup-wide staging), the four partial tiles summed through LDS in wave order
+// (deterministic), then bias / activation and the store.
+//
+// A vector-memory instruction costs the issuing wave some 30 cycles of matrix-core issue, so
+// their number per MFMA is what bounds the loop.  A fragments are one 16-byte load per lane
+// and 8-deep k block.  B fragments (lane (n, g) needs B[k][n] for four k) are four 4-byte
+// loads per block -- or, when B's rows allow 16-byte loads (BVEC), one: the wave fetches the
+// block's 8 x 32 sub-tile as 64 x 16 bytes, passes it through a private 1 KiB of LDS (LDS
+// instructions are almost free next to MFMAs) and reads its four values back.  512^3 gives 256 workgroups
 // instead of the 16 of the 64x256 tile; an N = 10 output layer
 // (MNIST/mnist_nn.cu:36-49) streams its activations once with row-clamped loads.
 //
@@ -16,13 +23,17 @@ namespace {
 constexpr int ST = 32;        // tile edge = one MFMA tile
 constexpr int RED_LD = 36;    // floats per row of a partial tile in LDS (16-byte rows, padded)
 
-template <bool HAS_BIAS, bool RELU>
+constexpr int BSTG_LD = 40;   // floats per k row of the B staging block: rows 4 apart (the two
+                              // halves of a wave) fall 32 banks apart
+
+template <bool HAS_BIAS, bool RELU, bool BVEC>
 __global__ __launch_bounds__(256) void f32_small_kernel(int M, int N, int K, int tiles_n,
                                                         const float* __restrict__ A, int64_t lda,
                                                         const float* __restrict__ B, int64_t ldb,
                                                         float* __restrict__ C, int64_t ldc,
                                                         const float* __restrict__ bias) {
   __shared__ __attribute__((aligned(16))) float red[4][ST][RED_LD];
+  __shared__ __attribute__((aligned(16))) float bstg[BVEC ? 4 : 1][BVEC ? 2 : 1][8][BSTG_LD];
   const int t = threadIdx.x;
   const int w = t >> 6, l = t & 63;
   const int r = l & 31, h = l >> 5;
@@ -42,18 +53,41 @@ __global__ __launch_bounds__(256) void f32_small_kernel(int M, int N, int K, int
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
-#pragma unroll 4
-  for (int b = b0; b < b1; ++b) {
+  // BVEC: lane l fetches B[8 b + l / 8][n0 + 4 (l % 8) .. + 3]; N is a multiple of 4 there, so a
+  // quad is inside or outside as a whole (outside: the last valid quad again, never stored)
+  const int vq = min(n0 + 4 * (l & 7), N - 4);
+  const float* bvp = B + (8 * (int64_t)b0 + (l >> 3)) * ldb + vq;
+  // one 8-deep k block: fragments in, four MFMAs
+  auto block = [&](int b) {
     const f32x4 a = *reinterpret_cast<const f32x4*>(ap);
-    const float x0 = bp[0], x1 = bp[ldb], x2 = bp[2 * ldb], x3 = bp[3 * ldb];
+    float x0, x1, x2, x3;
+    if (BVEC) {
+      float(*st)[BSTG_LD] = bstg[w][b & 1];
+      *reinterpret_cast<f32x4*>(&st[l >> 3][4 * (l & 7)]) = *reinterpret_cast<const f32x4*>(bvp);
+      // the same wave reads what it wrote: LDS serves a wave's instructions in order
+      x0 = st[4 * h][r], x1 = st[4 * h + 1][r], x2 = st[4 * h + 2][r], x3 = st[4 * h + 3][r];
+      bvp += 8 * ldb;
+    } else {
+      x0 = bp[0], x1 = bp[ldb], x2 = bp[2 * ldb], x3 = bp[3 * ldb];
+      bp += 8 * ldb;
+    }
     // (B fragment, A fragment): the lane then holds four consecutive columns of one row.
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x0, a[0], acc, 0, 0, 0);
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x1, a[1], acc, 0, 0, 0);
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x2, a[2], acc, 0, 0, 0);
     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x3, a[3], acc, 0, 0, 0);
     ap += 8;
-    bp += 8 * ldb;
+  };
+  int b = b0;
+  if (BVEC) {
+    // four blocks at a time, so that their loads are in flight together (with the strided
+    // B loads the plain loop measures 3 % faster)
+    for (; b + 4 <= b1; b += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) block(b + u);
+    }
   }
+  for (; b < b1; ++b) block(b);
 
   // acc[4q+e] is C[m0 + r][n0 + 8q + 4h + e].
 #pragma unroll
@@ -105,9 +139,17 @@ void launch_f32_small(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const
   const dim3 grid((unsigned)(tiles_m * (int64_t)tiles_n)), block(256);
   const float* bias = ba ? ba->bias : nullptr;
   const bool relu = ba && ba->relu;
-#define CIG_SMALL(HB, RL)                                                                   \
-  hipLaunchKernelGGL((f32_small_kernel<HB, RL>), grid, block, 0, ctx->stream, (int)M, (int)N, \
-                     (int)K, tiles_n, A, lda, B, ldb, C, ldc, bias)
+  // 16-byte loads of B's rows: every quad of columns whole and aligned
+  const bool bvec = N % 4 == 0 && ldb % 4 == 0 && (reinterpret_cast<uintptr_t>(B) & 15) == 0;
+#define CIG_SMALL(HB, RL)                                                                        \
+  do {                                                                                           \
+    if (bvec)                                                                                    \
+      hipLaunchKernelGGL((f32_small_kernel<HB, RL, true>), grid, block, 0, ctx->stream, (int)M,  \
+                         (int)N, (int)K, tiles_n, A, lda, B, ldb, C, ldc, bias);                 \
+    else                                                                                         \
+      hipLaunchKernelGGL((f32_small_kernel<HB, RL, false>), grid, block, 0, ctx->stream, (int)M, \
+                         (int)N, (int)K, tiles_n, A, lda, B, ldb, C, ldc, bias);                 \
+  } while (0)
   if (bias) {
     if (relu) CIG_SMALL(true, true); else CIG_SMALL(true, false);
   } else {
