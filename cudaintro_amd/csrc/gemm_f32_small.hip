@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void f32_small_kernel(int M, int N, int K, int
   auto block = [&](int b) {
     const f32x4 a = *reinterpret_cast<const f32x4*>(ap);
     float x0, x1, x2, x3;
-    if (BVEC) {
+    if constexpr (BVEC) {
       float(*st)[BSTG_LD] = bstg[w][b & 1];
       *reinterpret_cast<f32x4*>(&st[l >> 3][4 * (l & 7)]) = *reinterpret_cast<const f32x4*>(bvp);
       // the same wave reads what it wrote: LDS serves a wave's instructions in order
