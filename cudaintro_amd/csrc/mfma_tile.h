@@ -567,9 +567,9 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   int pslot = 0, next_pslot = 1, dma_pslot = 2;
   // One stage; PAR = its parity.  Single B stages: every stage issues B[s+3] and half of an A
   // pair: an even stage the first half of the pair of stages s+4, s+5 (its slot, one of three,
-  // has been free since the stage before), the odd stage after it the second half.  B pairs: even stages issue the A pair of stages
-  // s+4, s+5 (its slot, one of three, has been free since the stage before), odd stages the B
-  // pair of stages s+3, s+4 (its slot, one of two, is the one this stage stops reading): the
+  // has been free since the stage before), the odd stage after it the second half.  B pairs:
+  // even stages issue the A pair of stages s+4, s+5 (same slot rule), odd stages the B pair
+  // of stages s+3, s+4 (its slot, one of two, is the one this stage stops reading): the
   // instructions of a stage pair are spread over both of its stages.
   auto stage = [&](int s, auto par_const, auto steady_const) {
     constexpr int PAR = decltype(par_const)::value;
