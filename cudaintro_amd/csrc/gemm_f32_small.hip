@@ -9,8 +9,9 @@
 // and 8-deep k block.  B fragments (lane (n, g) needs B[k][n] for four k) are four 4-byte
 // loads per block -- or, when B's rows allow 16-byte loads (BVEC), one: the wave fetches the
 // block's 8 x 32 sub-tile as 64 x 16 bytes, passes it through a private 1 KiB of LDS (LDS
-// instructions are almost free next to MFMAs) and reads its four values back.  512^3 gives 256 workgroups
-// instead of the 16 of the 64x256 tile; an N = 10 output layer
+// instructions are almost free next to MFMAs) and reads its four values back.
+//
+// 512^3 gives 256 workgroups instead of the 16 of the 64x256 tile; an N = 10 output layer
 // (MNIST/mnist_nn.cu:36-49) streams its activations once with row-clamped loads.
 //
 // Ragged M and N: loads past the edge re-read the last valid row / column, stores are

@@ -371,7 +371,8 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   // single stages the K x N layouts use).
   constexpr bool BPAIR = BMODE == B_NK;
   constexpr int DMA_A = TILE_M / 8 / NW;        // per wave and stage pair: A instructions of 1 KiB
-  constexpr int DMA_B = (BPAIR ? 32 : 16) / NW; // per wave: B instructions per stage pair / per stage
+  // per wave: B instructions per stage pair (N x K weights) / per stage
+  constexpr int DMA_B = (BPAIR ? 32 : 16) / NW;
   constexpr int BPAIR_BYTES = 256 * 128;
   constexpr int APAIR_BYTES = TILE_M * 128;
   constexpr int B_RING = NSTAGES * OPERAND_BYTES;   // B slots first, then three A pair slots
@@ -457,7 +458,8 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
                  : "m0");
   };
   // d < DMA_B: B instruction d of stage `st` (of its stage pair, for N x K weights) into B
-  // slot `slot`; above: A instruction d - DMA_B of the stage pair st / 2 into pair slot `pslot`.  Past the last stage the last one is fetched
+  // slot `slot`; above: A instruction d - DMA_B of the stage pair st / 2 into pair slot `pslot`.
+  // Past the last stage the last one is fetched
   // again (into slots nobody reads any more), which keeps the number of outstanding
   // instructions, and so the vmcnt waits, uniform.
   // `steady_const`: the caller guarantees st < KTS and a pair that is not the odd tail, so
@@ -470,11 +472,13 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
       if (BPAIR) {
         uint32_t off = b_voff[d];
         if (tail_pair) off -= ((b_hi >> d) & 1u) << 6;
+        const int q = DMA_B * w + d;
         dma16(b_tile + (int64_t)(st >> 1) * 128, off,
-              lds_base + slot * BPAIR_BYTES + PairDma::dma_lds((DMA_B * w + d) >> 1, (DMA_B * w + d) & 1));
+              lds_base + slot * BPAIR_BYTES + PairDma::dma_lds(q >> 1, q & 1));
       } else {
+        const int q = DMA_B * w + d;
         dma16(b_tile + (int64_t)st * b_kstep, b_voff[d],
-              lds_base + slot * OPERAND_BYTES + BT::dma_lds((DMA_B * w + d) >> 2, (DMA_B * w + d) & 3));
+              lds_base + slot * OPERAND_BYTES + BT::dma_lds(q >> 2, q & 3));
       }
     } else {
       uint32_t off = a_voff[d - DMA_B];
@@ -653,7 +657,8 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
     stage(s, std::integral_constant<int, 0>{}, drain_t{});
     stage(s + 1, std::integral_constant<int, 1>{}, drain_t{});
   }
-  if (KTS & 1) stage(KTS - 1, std::integral_constant<int, 0>{}, drain_t{});  // odd stage count: the last one
+  // odd stage count: the last one
+  if (KTS & 1) stage(KTS - 1, std::integral_constant<int, 0>{}, drain_t{});
   wait_vmcnt(std::integral_constant<int, 0>{});  // no DMA outlives the main loop
   __syncthreads();  // ... for any wave, and every wave is done reading the ring
 
