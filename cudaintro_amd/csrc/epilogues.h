@@ -9,6 +9,12 @@
 //   out_row(row)             byte address of column 0 of that output row;
 //   operator()               pack + direct store (used where rows are not staged in LDS);
 //   shift_cols(c)            the same epilogue for the sub-problem starting at column c.
+// An epilogue whose row or column operand can be one word for the whole matrix (a per-tensor
+// scale) may declare `static constexpr bool HAS_UNIFORM_MODE = true` and give
+//   row_word(), col_word()           the address of that word (always readable);
+//   row_uniform(), col_uniform()     whether this call uses it;
+//   row_from_word(w), cols_from_word(w)   what load_row / load_cols would return, from it.
+// A kernel can then read the word once, with a scalar load, long before the epilogue.
 #pragma once
 
 #include <type_traits>
@@ -166,6 +172,13 @@ struct EpiDequantX4 {
   typedef typename std::conditional<OUT_BF16, u32x2, u32x4>::type packed_t;
   typedef float row_t;   // scale of the row
   typedef f32x4 col_t;   // scales of the four columns
+  static constexpr bool HAS_UNIFORM_MODE = true;
+  __device__ __forceinline__ const float* row_word() const { return sa; }
+  __device__ __forceinline__ const float* col_word() const { return sb; }
+  __device__ __forceinline__ bool row_uniform() const { return !sa_vec; }
+  __device__ __forceinline__ bool col_uniform() const { return !sb_vec; }
+  __device__ __forceinline__ row_t row_from_word(float w) const { return w; }
+  __device__ __forceinline__ col_t cols_from_word(float w) const { return f32x4{w, w, w, w}; }
   __device__ __forceinline__ row_t load_row(int64_t r) const { return sa[sa_vec ? r : 0]; }
   __device__ __forceinline__ col_t load_cols(int64_t c) const {
     if (sb_vec) return *reinterpret_cast<const f32x4*>(sb + c);

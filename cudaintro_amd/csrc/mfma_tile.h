@@ -334,6 +334,13 @@ struct EpiPartialX4 {
   __device__ __forceinline__ void side(int64_t, int64_t, T, T, T, T) const {}
   EpiPartialX4 shift_cols(int64_t c0) const { return EpiPartialX4{base + c0, ld, split_stride}; }
 };
+// An epilogue may declare `static constexpr bool HAS_UNIFORM_MODE = true` (see epilogues.h).
+template <typename E, typename = void>
+struct epi_has_uniform_mode : std::false_type {};
+template <typename E>
+struct epi_has_uniform_mode<E, typename std::enable_if<E::HAS_UNIFORM_MODE>::type>
+    : std::true_type {};
+
 // The epilogue of K range `split` (blockIdx.y): only the partial store depends on it.
 template <typename Epi>
 __device__ __forceinline__ Epi epilogue_of_split(const Epi& e, int) { return e; }
@@ -390,6 +397,13 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   tm = __builtin_amdgcn_readfirstlane(tm);
   tn = __builtin_amdgcn_readfirstlane(tn);
   const int64_t m0 = (int64_t)tm * TILE_M, n0 = (int64_t)tn * BN;
+  // Per-tensor operands of the epilogue: one word each at a uniform address, read here, before
+  // anything is written, hence with a scalar load whose latency nothing waits for.
+  float epi_row_word = 0.0f, epi_col_word = 0.0f;
+  if constexpr (epi_has_uniform_mode<Epi>::value) {
+    epi_row_word = *epi.row_word();
+    epi_col_word = *epi.col_word();
+  }
 
   // ---- DMA sources: uniform tile origin + per-lane byte offsets ------------------------------
   const char* a_tile = A + m0 * lda;  // + stage * KB
@@ -667,6 +681,12 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   // holds short pieces of 32 different rows.  Each wave stages one 32-row x 128-column block
   // at a time in its own piece of the (now idle) LDS and writes it out as whole rows: every
   // store instruction then covers full 256- or 512-byte row segments.
+  // The lane number as the epilogue sees it is opaque to the compiler, so that none of the
+  // epilogue's addresses is computed ahead and held in a register through the main loop.
+  int le = l;
+  asm volatile("" : "+v"(le));
+  le &= 63;
+  const int ge = le >> 5;
   constexpr int OB = Epi::OUT_BYTES;
   constexpr int ROW_BYTES = 128 * OB;
   constexpr int ROW_STRIDE = ROW_BYTES + 16;
@@ -680,28 +700,44 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   // What the epilogue needs per column quad (scales, bias) is the same for every row tile:
   // fetched once, up front, so that no load latency sits between the accumulator reads.
   typename Epi::col_t colv[4][4];
+  bool cols_done = false;
+  if constexpr (epi_has_uniform_mode<Epi>::value) {
+    if (epi.col_uniform()) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int64_t col = n0 + wn * 128 + 32 * j + 8 * q + 4 * g;
-      colv[j][q] = epi.load_cols(col < N ? col : N - 4);
+        for (int q = 0; q < 4; ++q) colv[j][q] = epi.cols_from_word(epi_col_word);
+      cols_done = true;
     }
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    const int64_t row0 = m0 + wm * 32 * MT + 32 * i;
-    const int64_t row = row0 + (l & 31);
-    const bool row_ok = row < M;
-    const int64_t row_c = row_ok ? row : M - 1;  // scale lookups stay in bounds
-    const typename Epi::row_t rowv = epi.load_row(row_c);
+  }
+  if (!cols_done) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int c = 32 * j + 8 * q + 4 * g;
+        const int64_t col = n0 + wn * 128 + 32 * j + 8 * q + 4 * ge;
+        colv[j][q] = epi.load_cols(col < N ? col : N - 4);
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const int64_t row0 = m0 + wm * 32 * MT + 32 * i;
+    const int64_t row = row0 + (le & 31);
+    const bool row_ok = row < M;
+    const int64_t row_c = row_ok ? row : M - 1;  // scale lookups stay in bounds
+    typename Epi::row_t rowv;
+    if constexpr (epi_has_uniform_mode<Epi>::value)
+      rowv = epi.row_uniform() ? epi.row_from_word(epi_row_word) : epi.load_row(row_c);
+    else
+      rowv = epi.load_row(row_c);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int c = 32 * j + 8 * q + 4 * ge;
         const int64_t col = n0 + wn * 128 + c;
         const bool col_ok = col < N;  // N is a multiple of 4: a quad is in or out as a whole
-        *reinterpret_cast<packed_t*>(scr + (l & 31) * ROW_STRIDE + c * OB) =
+        *reinterpret_cast<packed_t*>(scr + (le & 31) * ROW_STRIDE + c * OB) =
             epi.pack(rowv, colv[j][q], acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
                      acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
         if (row_ok && col_ok)
@@ -710,8 +746,8 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
       }
 #pragma unroll
     for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
-      const int rl = p * ROWS_PER_PASS + l / LANES_PER_ROW;
-      const int c16 = l % LANES_PER_ROW;
+      const int rl = p * ROWS_PER_PASS + le / LANES_PER_ROW;
+      const int c16 = le % LANES_PER_ROW;
       const u32x4 v = *reinterpret_cast<const u32x4*>(scr + rl * ROW_STRIDE + c16 * 16);
       // N * OB is a multiple of 16: a 16-byte piece is in or out as a whole
       if (row0 + rl < M && n0 + wn * 128 + c16 * (16 / OB) < N)

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256, 1) void mfma_probe_kernel(float* __restrict__ 
         facc4[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, x),
                                                           __builtin_bit_cast(f16x8, y), facc4[i], 0, 0, 0);
       else if (KIND == 6)
-        facc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, x[i & 3 ^ 1]),
+        facc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, x[(i & 3) ^ 1]),
                                                        __builtin_bit_cast(float, y[i & 3]), facc[i], 0, 0, 0);
       else
         iacc4[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, x),
