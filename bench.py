@@ -36,9 +36,22 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+SETTLE_SECONDS = 0.06
+
+
 def time_calls(torch, fn, steps, warmup):
     """W untimed calls, then exactly `steps` calls between a synchronize on both sides.
-    Returns (wall seconds, HIP-event seconds) for the timed region."""
+    Returns (wall seconds, HIP-event seconds) for the timed region.
+
+    Before the W warm-up calls the workload runs for SETTLE_SECONDS: each workload follows
+    host-side input generation, the GPU has idled meanwhile, and its clocks need some 30 ms of
+    work to leave the idle state (a 90 us kernel measured 8 % slow over its first 250
+    launches after two idle seconds, and at its steady rate from then on)."""
+    t_end = time.perf_counter() + SETTLE_SECONDS
+    while time.perf_counter() < t_end:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
