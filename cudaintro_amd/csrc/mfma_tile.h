@@ -545,7 +545,8 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   // MFMA m of a k-step: sub-step outermost, then column tile j, then row tile i: the first
   // MT need all A fragments (the first reads) but only the first pieces of B.
   auto mfma_piece = [&](const Frags& f, int m) {
-    const int sub = m / (4 * MT), j = (m % (4 * MT)) / MT, i = m % MT;
+    const int sub = m / (4 * MT), j = (m % (4 * MT)) / MT;
+    const int i = (j & 1) ? MT - 1 - m % MT : m % MT;   // back and forth: one operand stays
     if constexpr (BPAIR)
       acc[i][j] = Math::mfma(f.a[MT + j], Math::afrag(f.a[i], sub), acc[i][j]);
     else
