@@ -23,3 +23,12 @@ def test_gemm_common_header_names():
     for name in ("struct GemmResult", "run_gemm_bf16", "run_gemm_fp16", "run_gemm_fp32", "run_gemm_int8",
                  "const char* name;", "uint64_t iters;", "double secs;", "double tflops;"):
         assert name in text
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """`bench.py --gpus N` with N > 1 exits with a message before it touches the GPU."""
+    import sys
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                         capture_output=True, text=True, timeout=60)
+    assert out.returncode != 0
+    assert "one GPU" in (out.stdout + out.stderr)
