@@ -298,6 +298,14 @@ def main():
             per_config[f"fp32_{sz}"] = {"tflops": t, "frac_of_peak": t / PEAK_FP32_MATRIX_TFLOPS,
                                         "peak": PEAK_FP32_MATRIX_TFLOPS, "ms": e / steps * 1e3,
                                         "kernel": handle.last_kernel}
+            if sz == 512 and not args.no_cpu:
+                # the reference's own CPU check at its own size: matrixMulCPU, one thread
+                import oracle
+                t0 = time.perf_counter()
+                oracle.matrixMulCPU(Af, Bf)
+                dt = time.perf_counter() - t0
+                per_config["fp32_512"]["cpu_matrixMulCPU_one_thread_ms"] = dt * 1e3
+                per_config["fp32_512"]["cpu_gflops"] = wl.gemm_ops(sz, sz, sz) / dt / 1e9
 
         # MLP forward layers of the reference's MNIST demo on the fp32 GEMM with the fused
         # bias + ReLU epilogue (MNIST/mnist_nn.h:12-15: batch 20000, 784 -> 512 -> 10)
