@@ -322,6 +322,27 @@ def main():
                                 "peak": PEAK_FP32_MATRIX_TFLOPS, "ms": e / args.steps * 1e3,
                                 "kernel": handle.last_kernel}
 
+        # the steps either side of the int8 GEMM: device fills and the absmax row quantizer
+        # (HBM-bound; algorithmic bytes = what is written, resp. 4 + 1 bytes per element)
+        fb = torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda")
+        w_, e = time_calls(torch, lambda: handle.fill_random(fb, 0x1234), args.steps, args.warmup)
+        gbs = fb.numel() * 2 * args.steps / e / 1e9
+        per_config["fill_random_bf16_8192x8192"] = {"gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS,
+                                                    "peak": PEAK_HBM_GBS, "us": e / args.steps * 1e6,
+                                                    "bytes": fb.numel() * 2}
+        del fb
+        for rows_q, cols_q in ((2048, 4096), (8192, 8192)):
+            xq_ = torch.from_numpy(r.standard_normal((rows_q, cols_q)).astype(np.float32)).cuda()
+            outq = (torch.empty((rows_q, cols_q), dtype=torch.int8, device="cuda"),
+                    torch.empty((rows_q,), dtype=torch.float32, device="cuda"))
+            w_, e = time_calls(torch, lambda: handle.quantize_rows_i8(xq_, out=outq), args.steps, args.warmup)
+            nbytes = rows_q * cols_q * 5 + rows_q * 4
+            gbs = nbytes * args.steps / e / 1e9
+            per_config[f"quantize_rows_i8_{rows_q}x{cols_q}"] = {
+                "gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS, "peak": PEAK_HBM_GBS,
+                "us": e / args.steps * 1e6, "bytes": nbytes}
+            del xq_, outq
+
         # skinny decode shapes: HBM-bound.  Rotate over several distinct weight buffers so the
         # working set (> 256 MB) cannot sit in the Infinity Cache between calls.
         for M in (1, 8, 32):

@@ -321,12 +321,16 @@ class Handle:
         self._check(getattr(self.lib, name)(self._h, out.data_ptr(), out.numel(), seed, lo, hi), name)
         return out
 
-    def quantize_rows_i8(self, x):
+    def quantize_rows_i8(self, x, out=None):
         torch = _torch()
         assert x.dtype == torch.float32 and x.dim() == 2
         rows, cols = x.shape
-        q = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
-        s = torch.empty((rows,), dtype=torch.float32, device=x.device)
+        if out is None:
+            q = torch.empty((rows, cols), dtype=torch.int8, device=x.device)
+            s = torch.empty((rows,), dtype=torch.float32, device=x.device)
+        else:
+            q, s = out
+            assert q.dtype == torch.int8 and q.shape == x.shape and s.dtype == torch.float32
         st = self.lib.cigemm_quantize_rows_i8(self._h, rows, cols, x.data_ptr(), self._ld(x),
                                               q.data_ptr(), self._ld(q), s.data_ptr())
         self._check(st, "cigemm_quantize_rows_i8")

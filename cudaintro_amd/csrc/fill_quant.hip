@@ -5,8 +5,9 @@
 // GEMM_int8.cu:8-19).  Element idx depends only on (idx, seed), so the kernels are
 // written as grid-stride loops over 16-byte stores: HBM-write bound.
 //
-// quantize_rows_i8: one workgroup per row, two passes over the row (absmax, then
-// scale+round); the row is read twice from L2/HBM and written once.
+// quantize_rows_i8: one workgroup per row, absmax then scale+round.  Rows of whole 16-byte
+// pieces up to 16384 columns are held in registers between the two (read once, 16-byte
+// loads, 4-byte stores); any other row is read twice, element by element.
 #include "common.h"
 
 namespace cig {
@@ -108,6 +109,59 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(int64_t cols,
   }
 }
 
+// The same for rows of whole 16-byte pieces (cols a multiple of 4, aligned rows) of up to
+// 1024 * CHUNKS columns: a lane keeps its CHUNKS pieces of the row in registers, so the row is
+// read once, as 16-byte loads, and written as packed 4-byte stores.  Same arithmetic per
+// element as the kernel above (the maximum does not depend on the order it is taken in).
+template <int CHUNKS>
+__global__ __launch_bounds__(256) void quantize_rows_vec_kernel(int64_t cols,
+                                                                const float* __restrict__ x,
+                                                                int64_t ldx,
+                                                                int8_t* __restrict__ q,
+                                                                int64_t ldq,
+                                                                float* __restrict__ scale) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const f32x4* xr = reinterpret_cast<const f32x4*>(x + row * ldx);
+  uint32_t* qr = reinterpret_cast<uint32_t*>(q + row * ldq);
+  const int nquad = (int)(cols >> 2);
+  f32x4 v[CHUNKS];
+  float amax = 0.0f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    v[c] = i < nquad ? xr[i] : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) amax = fmaxf(amax, fabsf(v[c][e]));
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float s = amax > 0.0f ? __fdiv_rn(amax, 127.0f) : 1.0f;
+  if (threadIdx.x == 0) scale[row] = s;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = threadIdx.x + 256 * c;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float r = rintf(__fdiv_rn(v[c][e], s));  // ties to even
+      r = fminf(fmaxf(r, -127.0f), 127.0f);
+      packed |= ((uint32_t)(int)r & 0xffu) << (8 * e);
+    }
+    if (i < nquad) qr[i] = packed;
+  }
+}
+
+template <int CHUNKS>
+void launch_quantize_vec(cigemmContext* ctx, int64_t rows, int64_t cols, const float* x,
+                         int64_t ldx, int8_t* q, int64_t ldq, float* scale) {
+  hipLaunchKernelGGL((quantize_rows_vec_kernel<CHUNKS>), dim3((unsigned)rows), dim3(256), 0,
+                     ctx->stream, cols, x, ldx, q, ldq, scale);
+}
+
 }  // namespace
 }  // namespace cig
 
@@ -172,8 +226,21 @@ cigemmStatus_t cigemm_quantize_rows_i8(cigemmHandle_t h, int64_t rows, int64_t c
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "cigemm_quantize_rows_i8: ld < cols");
   if (rows > 2147483647LL)
     return fail(h, CIGEMM_STATUS_NOT_SUPPORTED, "cigemm_quantize_rows_i8: rows > 2^31-1");
-  hipLaunchKernelGGL(quantize_rows_kernel, dim3((unsigned)rows), dim3(256), 0, h->stream, cols, x,
-                     ldx, q, ldq, scale);
+  const bool pieces = cols > 0 && cols % 4 == 0 && ldx % 4 == 0 && ldq % 4 == 0 &&
+                      ((uintptr_t)x & 15) == 0 && ((uintptr_t)q & 3) == 0 && cols <= 16384;
+  if (pieces && cols <= 1024)
+    launch_quantize_vec<1>(h, rows, cols, x, ldx, q, ldq, scale);
+  else if (pieces && cols <= 2048)
+    launch_quantize_vec<2>(h, rows, cols, x, ldx, q, ldq, scale);
+  else if (pieces && cols <= 4096)
+    launch_quantize_vec<4>(h, rows, cols, x, ldx, q, ldq, scale);
+  else if (pieces && cols <= 8192)
+    launch_quantize_vec<8>(h, rows, cols, x, ldx, q, ldq, scale);
+  else if (pieces)
+    launch_quantize_vec<16>(h, rows, cols, x, ldx, q, ldq, scale);
+  else
+    hipLaunchKernelGGL(quantize_rows_kernel, dim3((unsigned)rows), dim3(256), 0, h->stream, cols,
+                       x, ldx, q, ldq, scale);
   return check_launch(h, "cigemm_quantize_rows_i8");
 }
 

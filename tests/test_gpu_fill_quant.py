@@ -69,7 +69,8 @@ def test_fill_unaligned_and_other_range(handle, torch_gpu, oracle):
     assert got[0] == 0
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 300), (257, 4096), (2048, 4096)])
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 300), (257, 4096), (2048, 4096), (7, 1028),
+                                   (4, 2052), (5, 8192), (3, 16384), (2, 16388), (3, 4098)])
 def test_quantize_rows(handle, torch_gpu, oracle, rng, shape):
     x = rng.normal(size=shape).astype(np.float32)
     x[0] = 0.0   # zero row
@@ -77,5 +78,18 @@ def test_quantize_rows(handle, torch_gpu, oracle, rng, shape):
         x[-1, :4] = [1.5, -1.5, 3.0, -3.0]
     q, s = handle.quantize_rows_i8(torch_gpu.from_numpy(x).cuda())
     qe, se = oracle.quantize_rows_i8(x)
+    np.testing.assert_array_equal(s.cpu().numpy(), se)
+    np.testing.assert_array_equal(q.cpu().numpy(), qe)
+
+
+@pytest.mark.parametrize("pad", [4, 1])
+def test_quantize_rows_of_a_wider_matrix(handle, torch_gpu, oracle, rng, pad):
+    """Rows with a leading dimension above the column count: a multiple of 4 keeps the
+    16-byte-piece kernel, any other falls back to the element-wise one; same bits."""
+    rows, cols = 33, 1024
+    wide = rng.normal(size=(rows, cols + pad)).astype(np.float32) * 3
+    xd = torch_gpu.from_numpy(wide).cuda()[:, :cols]
+    q, s = handle.quantize_rows_i8(xd)
+    qe, se = oracle.quantize_rows_i8(np.ascontiguousarray(wide[:, :cols]))
     np.testing.assert_array_equal(s.cpu().numpy(), se)
     np.testing.assert_array_equal(q.cpu().numpy(), qe)
