@@ -32,3 +32,15 @@ def test_bench_refuses_more_than_one_gpu():
                          capture_output=True, text=True, timeout=60)
     assert out.returncode != 0
     assert "one GPU" in (out.stdout + out.stderr)
+
+
+def test_fill_kernels_division_free_forms_are_exact(tmp_path):
+    """The device fills replace the IEEE division by 2^24 - 1 and the integer modulo by
+    multiply-based forms; this checks them against the plain expressions for every operand."""
+    exe = tmp_path / "test_exact_arith"
+    subprocess.run(["gcc", "-O2", "-std=c11", "-ffp-contract=off", "-Wall",
+                    os.path.join(ROOT, "tests", "cpp", "test_exact_arith.c"), "-o", str(exe), "-lm"],
+                   check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "exact arithmetic OK" in out.stdout
