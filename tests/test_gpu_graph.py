@@ -67,3 +67,39 @@ def test_gemm_sequence_replays_from_a_graph(torch_gpu, oracle, rng):
             assert torch.equal(o.view(torch.int16) if o.dtype == torch.bfloat16 else o,
                                e.view(torch.int16) if e.dtype == torch.bfloat16 else e), (replay, k, names[k])
     h.close()
+
+
+def test_two_handles_on_two_streams_do_not_share_state(torch_gpu, oracle, rng):
+    """One handle per stream: each owns its split-K workspace and arrival counters, so the two
+    streams can run split-K calls at the same time.  Forty calls alternate between the streams
+    without a synchronisation in between; every output equals the one computed alone."""
+    torch = torch_gpu
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    handles = [ci.Handle(stream=s) for s in streams]
+
+    def bf(shape, scale=1.0):
+        return to_dev(torch, oracle.f32_to_bf16((scale * rng.standard_normal(shape)).astype(np.float32)), "bf16")
+
+    # a skinny call (fix-up inside the kernel) and a split-K tile call (two launches) per stream
+    work = []
+    for _ in streams:
+        work.append([(bf((8, 4096)), bf((4096, 1024), 0.05)), (bf((64, 4096)), bf((4096, 1024), 0.05))])
+    torch.cuda.synchronize()
+    alone = []
+    for h, s, jobs in zip(handles, streams, work):
+        with torch.cuda.stream(s):
+            alone.append([h.gemm_bf16(a, b).clone() for a, b in jobs])
+        s.synchronize()
+    assert "skinny" in handles[0].last_kernel or "splitk" in handles[0].last_kernel
+    outs = [[torch.empty_like(o) for o in res] for res in alone]
+    for rep in range(20):
+        for i, (h, s, jobs) in enumerate(zip(handles, streams, work)):
+            with torch.cuda.stream(s):
+                for (a, b), o in zip(jobs, outs[i]):
+                    h.gemm_bf16(a, b, out=o)
+    torch.cuda.synchronize()
+    for res, got in zip(alone, outs):
+        for r, g in zip(res, got):
+            assert torch.equal(r.view(torch.int16), g.view(torch.int16))
+    for h in handles:
+        h.close()
