@@ -321,6 +321,11 @@ def main():
             per_config[name] = {"tflops": t, "frac_of_peak": t / PEAK_FP32_MATRIX_TFLOPS,
                                 "peak": PEAK_FP32_MATRIX_TFLOPS, "ms": e / args.steps * 1e3,
                                 "kernel": handle.last_kernel}
+            if Nb <= 16:   # a narrow output layer streams its activations: HBM is the bound
+                nbytes = 4 * (Mb * Kb + Kb * Nb + Mb * Nb + Nb)
+                gbs = nbytes * args.steps / e / 1e9
+                per_config[name].update({"gbs": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS,
+                                         "bytes": nbytes})
 
         # the steps either side of the int8 GEMM: device fills and the absmax row quantizer
         # (HBM-bound; algorithmic bytes = what is written, resp. 4 + 1 bytes per element)

@@ -165,6 +165,66 @@ def test_small_kernel_ragged_shapes(handle, torch_gpu, oracle, rng, shape, pad_c
     assert "small" in name, name
 
 
+@pytest.mark.parametrize("shape", [(64, 1, 16), (65, 3, 48), (1000, 10, 784), (20000, 10, 512), (333, 16, 2048),
+                                   (127, 13, 1040), (4097, 7, 32)])
+@pytest.mark.parametrize("pad_cols", [4, 1])
+def test_narrow_kernel_ragged_shapes(handle, torch_gpu, oracle, rng, shape, pad_cols):
+    """N <= 16, K a multiple of 16 up to 2048, M >= 64: the 16x16 form of the small kernel
+    (each wave keeps its share of B in registers); guard rows / columns stay untouched."""
+    name = ragged_check(handle, torch_gpu, oracle, rng, ci.ALGO_SMALL, shape, pad_cols)
+    assert "small_16x16" in name, name
+
+
+@pytest.mark.parametrize("shape", [(63, 10, 512), (1000, 17, 512), (1000, 10, 2064), (1000, 10, 520)])
+def test_narrow_kernel_gate(handle, torch_gpu, oracle, rng, shape):
+    """Just outside the 16x16 form's conditions (M, N, K share per wave, K % 16) the 32x32
+    form runs."""
+    name = ragged_check(handle, torch_gpu, oracle, rng, ci.ALGO_SMALL, shape)
+    assert "small_32x32" in name, name
+
+
+def test_narrow_kernel_onehot_bias_relu(handle, torch_gpu, oracle, rng):
+    """One-hot operands pick single elements (every index of the fragment layout), exact
+    inputs make bias + ReLU comparable bit for bit."""
+    torch = torch_gpu
+    M, N, K = 200, 10, 784
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    X = rng.choice(vals, size=(M, K))
+    Wm = np.zeros((K, N), np.float32)
+    ks = rng.integers(0, K, size=N)
+    Wm[ks, np.arange(N)] = 1.0                      # column n copies column ks[n] of X
+    with handle.algo(ci.ALGO_SMALL):
+        out = handle.gemm_f32(torch.from_numpy(X).cuda(), torch.from_numpy(Wm).cuda()).cpu().numpy()
+        assert "small_16x16" in handle.last_kernel
+        np.testing.assert_array_equal(out, X[:, ks])
+        Wd = rng.choice(vals, size=(K, N))
+        bias = rng.choice(vals, size=N)
+        L = handle.linear_f32(torch.from_numpy(X).cuda(), torch.from_numpy(Wd).cuda(),
+                              torch.from_numpy(bias).cuda(), ci.ACT_RELU).cpu().numpy()
+        assert "small_16x16" in handle.last_kernel
+    np.testing.assert_array_equal(L, oracle.linear_f32(X, Wd, bias, True))
+
+
+def test_narrow_kernel_weights_inside_a_wider_matrix(handle, torch_gpu, oracle, rng):
+    """Contiguous, aligned weights pass through LDS as 16-byte pieces; a column slice of a
+    wider matrix (other leading dimension, unaligned start) is read element by element.
+    Both give the same bits."""
+    torch = torch_gpu
+    M, N, K = 500, 10, 512
+    X = rng.uniform(-1, 1, size=(M, K)).astype(np.float32)
+    wide = rng.uniform(-1, 1, size=(K, 24)).astype(np.float32)
+    Wc = np.ascontiguousarray(wide[:, 3:3 + N])
+    xd, wd = torch.from_numpy(X).cuda(), torch.from_numpy(wide).cuda()
+    with handle.algo(ci.ALGO_SMALL):
+        a = handle.gemm_f32(xd, torch.from_numpy(Wc).cuda()).cpu().numpy()
+        assert "small_16x16" in handle.last_kernel
+        b = handle.gemm_f32(xd, wd[:, 3:3 + N]).cpu().numpy()
+        assert "small_16x16" in handle.last_kernel
+    np.testing.assert_array_equal(a, b)
+    ref, S = oracle.gemm_f64(X, Wc, with_abs=True)
+    assert (np.abs(a - ref) <= K * 2.0 ** -24 * S + 1e-30).all()
+
+
 def test_default_choice_by_shape(handle, torch_gpu):
     """Small problems and narrow outputs go to the 32x32 kernel, large ones to 256-column
     tiles, what neither takes to the any-shape kernel."""
@@ -175,7 +235,7 @@ def test_default_choice_by_shape(handle, torch_gpu):
     assert handle.get_algo() == ci.ALGO_DEFAULT
     assert "small" in kernel_for(512, 512, 512)
     assert "small" in kernel_for(1024, 1024, 1024)
-    assert "small" in kernel_for(20000, 10, 512)
+    assert "small_16x16" in kernel_for(20000, 10, 512)
     assert "mfma_256" in kernel_for(2048, 2048, 2048)
     assert "mfma_256" in kernel_for(4096, 4096, 64)
     assert "mfma_256" in kernel_for(20000, 512, 784)
