@@ -17,6 +17,9 @@
 // workspace, then bumps a per-column-slab counter; the workgroup that finds it is the last
 // one sums the partials in split order (so the result does not depend on arrival order),
 // applies the epilogue and resets the counter.
+//
+// int8 weights with at least one 32-column slab per compute unit take a second kernel that
+// needs none of that: K is split over the four waves of the workgroup (further down).
 #include "epilogues.h"
 #include "mfma_tile.h"
 
@@ -60,14 +63,22 @@ struct GeoKN16 {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       dma16(W + WT::dma_src(w, i, l, ldw, 31), slot_lds + WT::dma_lds(w, i));
+    // x: only the groups of four rows that hold a row below M (the other rows of the padded
+    // tile keep whatever the LDS holds: their products are never stored)
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int r = 8 * w + 4 * i + (l >> 4);
-      const int rr = r < M ? r : M - 1;
-      const int chunk = ((l & 15) >> 2) ^ tile::rowmajor_swz(r);
-      dma4(x + (int64_t)rr * ldx + (chunk << 4) + ((l & 3) << 2),
-           slot_lds + W_BYTES + (8 * w + 4 * i) * 64);
+      if (8 * w + 4 * i < M) {
+        const int r = 8 * w + 4 * i + (l >> 4);
+        const int rr = r < M ? r : M - 1;
+        const int chunk = ((l & 15) >> 2) ^ tile::rowmajor_swz(r);
+        dma4(x + (int64_t)rr * ldx + (chunk << 4) + ((l & 3) << 2),
+             slot_lds + W_BYTES + (8 * w + 4 * i) * 64);
+      }
     }
+  }
+  // DMA instructions wave w issues per stage
+  static __device__ __forceinline__ int dma_count(int M, int w) {
+    return 4 + (8 * w < M ? 1 : 0) + (8 * w + 4 < M ? 1 : 0);
   }
   static __device__ __forceinline__ void compute(const char* slot, int w, int l,
                                                  typename Math::acc_t (&acc)[NT]) {
@@ -115,10 +126,14 @@ struct GeoNK8 {
       const int r = 32 * w + 8 * i + (l >> 3);
       dma16(W + (int64_t)r * ldw + (((l & 7) ^ swz(r)) << 4), slot_lds + (32 * w + 8 * i) * 128);
     }
-    const int r = 8 * w + (l >> 3);
-    const int rr = r < M ? r : M - 1;
-    dma16(x + (int64_t)rr * ldx + (((l & 7) ^ swz(r)) << 4), slot_lds + W_BYTES + (8 * w) * 128);
+    // x: only the groups of eight rows that hold a row below M (see above)
+    if (8 * w < M) {
+      const int r = 8 * w + (l >> 3);
+      const int rr = r < M ? r : M - 1;
+      dma16(x + (int64_t)rr * ldx + (((l & 7) ^ swz(r)) << 4), slot_lds + W_BYTES + (8 * w) * 128);
+    }
   }
+  static __device__ __forceinline__ int dma_count(int M, int w) { return 4 + (8 * w < M ? 1 : 0); }
   static __device__ __forceinline__ void compute(const char* slot, int w, int l,
                                                  Math::acc_t (&acc)[NT]) {
     const char* sx = slot + W_BYTES;
@@ -222,11 +237,18 @@ __global__ __launch_bounds__(256, 1) void skinny_kernel(int M, int N, int stages
 #pragma unroll
   for (int st = 0; st < DIST; ++st) issue(st, st);
 
+  // this wave's DMA instructions per stage: the W pieces plus the x pieces below row M
+  const int dps = Geo::dma_count(M, w);
   int slot = 0, dma_slot = DIST;
   for (int s = 0; s < KTS; ++s) {
     // stage s landed for this wave (stages s+1 .. s+DIST-1 may be in flight); after the barrier
     // it is visible to all waves and every wave has finished reading stage s-1
-    wait_vmcnt(std::integral_constant<int, DPS*(DIST - 1)>{});
+    if (dps == DPS)
+      wait_vmcnt(std::integral_constant<int, DPS*(DIST - 1)>{});
+    else if (dps == DPS - 1)
+      wait_vmcnt(std::integral_constant<int, (DPS - 1) * (DIST - 1)>{});
+    else
+      wait_vmcnt(std::integral_constant<int, (DPS - 2) * (DIST - 1)>{});
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     issue(s + DIST, dma_slot);
@@ -335,6 +357,160 @@ void launch_skinny(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const vo
   }
 }
 
+// ---- int8, N x K weights, many columns: no split-K ------------------------------------------
+// With at least one 32-column slab per compute unit the K split moves inside the workgroup:
+// a stage is 512 k of the slab's 32 weight rows (16 KiB, 512 contiguous bytes per row) plus
+// the same 512 k of XR rows of x (XR = 8, 16 or 32, the smallest that holds M); wave w moves
+// and multiplies k-chunk w (128 k) of every stage, and the four partial 32 x 32 tiles are
+// summed through LDS in wave order at the end.  No partials in memory, no arrival counter, no
+// second pass: the three dependent trips through the fabric that the split-K fix-up costs
+// (about 5 us per call) are gone.
+template <int XR_>
+struct NK8KW {
+  static constexpr int BN = 32;
+  static constexpr int K_ELEMS = 512;
+  static constexpr int XR = XR_;                     // rows of x held per stage
+  static constexpr int W_BYTES = 32 * 512;           // four [32 n][128 B] sub-tiles, one per wave
+  static constexpr int X_BYTES = XR * 512;           // four [XR m][128 B] sub-tiles
+  static constexpr int STAGE_BYTES = W_BYTES + X_BYTES;
+  static constexpr int NSTAGES = XR == 8 ? 7 : XR == 16 ? 6 : 5;   // 140 / 144 / 160 KiB
+  static constexpr int DPS = 4 + XR / 8;             // per wave and stage, 1 KiB each
+};
+
+template <typename Epi, int XR>
+__global__ __launch_bounds__(256, 1) void skinny_nk8_kwaves_kernel(int M, int N, int KTS,
+                                                                   const char* __restrict__ X,
+                                                                   int64_t ldx,
+                                                                   const char* __restrict__ W,
+                                                                   int64_t ldw, Epi epi) {
+  typedef tile::MathI8 Math;
+  typedef NK8KW<XR> G;
+  constexpr int NS = G::NSTAGES, DIST = NS - 1;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int t = threadIdx.x, l = t & 63;
+  const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int64_t n0 = (int64_t)blockIdx.x * G::BN;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+
+  // this lane's DMA sources of stage 0: row 8 i + l / 8 of the slab (i = 0..3) and of x
+  // (i < XR / 8; rows >= M re-read row M - 1), 16-byte chunk (l % 8) ^ swz(row) of k-chunk w
+  const char* wsrc[4];
+  const char* xsrc[XR / 8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 8 * i + (l >> 3);
+    wsrc[i] = W + (n0 + r) * ldw + 128 * w + (((l & 7) ^ GeoNK8::swz(r)) << 4);
+    if (i < XR / 8)
+      xsrc[i] = X + (int64_t)(r < M ? r : M - 1) * ldx + 128 * w + (((l & 7) ^ GeoNK8::swz(r)) << 4);
+  }
+  // Workgroups start at different stages of K and wrap around (integer sums do not depend on
+  // the order): at any moment they read different 512-byte columns of their rows, which spreads
+  // the requests over the memory channels (19.4 -> 14.1 us per call at N = K = 8192).
+  const int rot = (int)((blockIdx.x * 7u) % (unsigned)KTS);
+  auto issue = [&](int st, int slot) {
+    st = st < KTS ? st : KTS - 1;  // past the end: refetch the last stage into a dead slot
+    st += rot;
+    st = st < KTS ? st : st - KTS;
+    const uint32_t dst = lds_base + slot * G::STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      dma16(wsrc[i] + (int64_t)st * G::K_ELEMS, dst + w * 4096 + (8 * i) * 128);
+#pragma unroll
+    for (int i = 0; i < XR / 8; ++i)
+      dma16(xsrc[i] + (int64_t)st * G::K_ELEMS, dst + G::W_BYTES + w * (XR * 128) + (8 * i) * 128);
+  };
+  auto wait_vmcnt = [](auto n_const) {
+    constexpr int n = decltype(n_const)::value;
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+  };
+
+  Math::acc_t acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0;
+#pragma unroll
+  for (int st = 0; st < DIST; ++st) issue(st, st);
+
+  int slot = 0, dma_slot = DIST;
+  for (int s = 0; s < KTS; ++s) {
+    // Stage s landed for this wave.  No workgroup barrier: a wave reads only the k-chunk it
+    // moved itself, and the slot it refills now is the one of stage s - 1, whose fragments
+    // its own MFMAs have already consumed.
+    wait_vmcnt(std::integral_constant<int, G::DPS*(DIST - 1)>{});
+    __builtin_amdgcn_sched_barrier(0);
+    issue(s + DIST, dma_slot);
+    const char* sw = lds + slot * G::STAGE_BYTES + w * 4096;
+    const char* sx = lds + slot * G::STAGE_BYTES + G::W_BYTES + w * (XR * 128);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      // rows XR .. 31 of the padded x tile alias rows 0 .. XR - 1: never stored
+      const u32x4 xf =
+          *reinterpret_cast<const u32x4*>(sx + GeoNK8::off(l & (XR - 1), 2 * kk + (l >> 5)));
+      const u32x4 wf = *reinterpret_cast<const u32x4*>(sw + GeoNK8::off(l & 31, 2 * kk + (l >> 5)));
+      acc = Math::mfma(wf, xf, acc);
+    }
+    slot = slot + 1 == NS ? 0 : slot + 1;
+    dma_slot = dma_slot + 1 == NS ? 0 : dma_slot + 1;
+  }
+  wait_vmcnt(std::integral_constant<int, 0>{});
+  __syncthreads();  // no DMA in flight, every wave done reading: the ring can be reused
+
+  // acc[4 q + e] = partial of y[l % 32][n0 + 8 q + 4 (l / 32) + e] over this wave's k-chunks
+  int32_t* red = reinterpret_cast<int32_t*>(lds);  // [4 waves][32 m][36]
+  constexpr int RLD = 36;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const i32x4 v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+    *reinterpret_cast<i32x4*>(red + (w * 32 + (l & 31)) * RLD + 8 * q + 4 * (l >> 5)) = v;
+  }
+  __syncthreads();
+  const int m = t >> 3, c = (t & 7) * 4;
+  if (m >= M) return;
+  i32x4 sum = *reinterpret_cast<const i32x4*>(red + m * RLD + c);
+#pragma unroll
+  for (int ww = 1; ww < 4; ++ww) {
+    const i32x4 p = *reinterpret_cast<const i32x4*>(red + (ww * 32 + m) * RLD + c);
+    sum += p;
+  }
+  epi(m, n0 + c, sum[0], sum[1], sum[2], sum[3]);
+}
+
+template <typename Epi, int XR>
+void launch_skinny_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
+                          int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
+  typedef NK8KW<XR> G;
+  constexpr int LDS_BYTES = G::NSTAGES * G::STAGE_BYTES;
+  static_assert(LDS_BYTES <= 160 * 1024, "ring must fit the LDS");
+  auto kern = skinny_nk8_kwaves_kernel<Epi, XR>;
+  static int attr_device = -1;
+  if (attr_device != ctx->device) {
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              LDS_BYTES);
+    attr_device = ctx->device;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN)), dim3(256), LDS_BYTES, ctx->stream, (int)M,
+                     (int)N, (int)(K / G::K_ELEMS), static_cast<const char*>(X), ldx_bytes,
+                     static_cast<const char*>(W), ldw_bytes, epi);
+}
+
+// int8 N x K: the kernel above when it applies (a slab per compute unit, K in whole 512-k
+// stages), else the split-K kernel.  Returns true when the first one ran.
+template <typename Epi>
+bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
+                       int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  if (K % 512 == 0 && N % 32 == 0 && N / 32 >= cus) {
+    if (M <= 8)
+      launch_skinny_kwaves<Epi, 8>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    else if (M <= 16)
+      launch_skinny_kwaves<Epi, 16>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    else
+      launch_skinny_kwaves<Epi, 32>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    return true;
+  }
+  launch_skinny<GeoNK8>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+  return false;
+}
+
 template <typename Geo>
 bool skinny_shape_ok(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K, int elem,
                      const void* X, int64_t ldx, const void* W, int64_t ldw) {
@@ -373,8 +549,8 @@ bool launch_skinny_i8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const
   if (!skinny_shape_ok<GeoNK8>(ctx, M, N, K, 1, A, lda, B, ldb)) return false;
   if (!dq) {
     if (ldc % 4 || ((uintptr_t)C & 15)) return false;
-    launch_skinny<GeoNK8>(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32x4{C, ldc});
-    ctx->last_kernel = "i8_skinny_32x128_ring7_nk";
+    const bool kw = launch_skinny_nk8(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32x4{C, ldc});
+    ctx->last_kernel = kw ? "i8_skinny_32x32_kwaves_nk" : "i8_skinny_32x128_ring7_nk";
     return true;
   }
   if (dq->out_bf16 ? (dq->ldo % 4 || ((uintptr_t)dq->out & 7))
@@ -383,17 +559,18 @@ bool launch_skinny_i8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const
   if (dq->sb_vec && ((uintptr_t)dq->sb & 15)) return false;
   if (dq->acc_out && (dq->ldacc % 4 || ((uintptr_t)dq->acc_out & 15))) return false;
 #define CIG_DQ(OB, DA)                                                                          \
-  launch_skinny<GeoNK8>(ctx, M, N, K, A, lda, B, ldb,                                           \
-                        EpiDequantX4<OB, DA>{dq->out, dq->ldo, dq->sa, dq->sb, dq->sa_vec,      \
-                                             dq->sb_vec, dq->acc_out, dq->ldacc})
+  launch_skinny_nk8(ctx, M, N, K, A, lda, B, ldb,                                               \
+                    EpiDequantX4<OB, DA>{dq->out, dq->ldo, dq->sa, dq->sb, dq->sa_vec,          \
+                                         dq->sb_vec, dq->acc_out, dq->ldacc})
   const bool dump = dq->acc_out != nullptr;
+  bool kw;
   if (dq->out_bf16) {
-    if (dump) CIG_DQ(true, true); else CIG_DQ(true, false);
+    kw = dump ? CIG_DQ(true, true) : CIG_DQ(true, false);
   } else {
-    if (dump) CIG_DQ(false, true); else CIG_DQ(false, false);
+    kw = dump ? CIG_DQ(false, true) : CIG_DQ(false, false);
   }
 #undef CIG_DQ
-  ctx->last_kernel = "i8_skinny_32x128_ring7_nk_dequant";
+  ctx->last_kernel = kw ? "i8_skinny_32x32_kwaves_nk_dequant" : "i8_skinny_32x128_ring7_nk_dequant";
   return true;
 }
 

@@ -95,6 +95,39 @@ def test_skinny_int8_nk(handle, torch_gpu, oracle, rng, M, N, K, out_type):
     np.testing.assert_array_equal(got, expect)
 
 
+@pytest.mark.parametrize("M", [1, 5, 8, 9, 16, 17, 32])
+@pytest.mark.parametrize("N,K", [(8192, 512), (8192 + 128, 1536), (8192, 4096 + 128)])
+def test_skinny_int8_without_split_k(handle, torch_gpu, oracle, rng, M, N, K):
+    """A 32-column slab per compute unit and K in whole 512-k stages: the kernel that splits K
+    over the waves of a workgroup instead of over workgroups, with 8, 16 or 32 rows of x per
+    stage.  Outside those conditions (K = 4224) the split-K kernel runs; same bits either way."""
+    torch = torch_gpu
+    if torch.cuda.get_device_properties(0).multi_processor_count > 256:
+        pytest.skip("the shapes assume at most 256 compute units")
+    X = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    acc_ref = oracle.gemm_i8_i32(X, W, b_is_nk=True)
+    xd, wd = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda()
+    expect_kw = K % 512 == 0
+    out = torch.full((M + 2, N + 4), -9, dtype=torch.int32, device="cuda")
+    for _ in range(2):
+        handle.gemm_i8_i32(xd, wd, ci.B_NK, out=out[:M, :N])
+        assert ("kwaves" in handle.last_kernel) == expect_kw, handle.last_kernel
+        o = out.cpu().numpy()
+        np.testing.assert_array_equal(o[:M, :N], acc_ref)
+        assert (o[M:] == -9).all() and (o[:, N:] == -9).all()
+    sa = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
+    sb = rng.uniform(1e-3, 5e-2, N).astype(np.float32)
+    for out_type, ot in (("f32", ci.OUT_F32), ("bf16", ci.OUT_BF16)):
+        y, acc = handle.gemm_i8_dequant(xd, wd, torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda(),
+                                        ci.B_NK, ot, dump_acc=True)
+        assert ("kwaves" in handle.last_kernel) == expect_kw, handle.last_kernel
+        np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
+        expect = oracle.dequant(acc_ref, sa, sb, out_dtype=out_type, sa_per_row=M > 1, sb_per_col=True)
+        got = bits(torch, y) if out_type == "bf16" else y.cpu().numpy()
+        np.testing.assert_array_equal(got, expect)
+
+
 def test_config_skinny_decode(handle, torch_gpu, oracle):
     """The decode-shaped configurations: M in {1, 8, 32}, N = K = 8192, bf16 weights N(0,0.02)
     and int8 weights with per-channel scales."""
