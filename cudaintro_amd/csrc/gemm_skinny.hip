@@ -378,7 +378,7 @@ struct NK8KW {
 };
 
 template <typename Epi, int XR>
-__global__ __launch_bounds__(256, 1) void skinny_nk8_kwaves_kernel(int M, int N, int KTS,
+__global__ __launch_bounds__(256, 1) void skinny_nk8_kwaves_kernel(int M, int N, int K,
                                                                    const char* __restrict__ X,
                                                                    int64_t ldx,
                                                                    const char* __restrict__ W,
@@ -391,33 +391,42 @@ __global__ __launch_bounds__(256, 1) void skinny_nk8_kwaves_kernel(int M, int N,
   const int w = __builtin_amdgcn_readfirstlane(t >> 6);
   const int64_t n0 = (int64_t)blockIdx.x * G::BN;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  // K is a multiple of 128: the last stage may hold fewer than four k-chunks
+  const int KTS = (K + G::K_ELEMS - 1) / G::K_ELEMS;
 
-  // this lane's DMA sources of stage 0: row 8 i + l / 8 of the slab (i = 0..3) and of x
-  // (i < XR / 8; rows >= M re-read row M - 1), 16-byte chunk (l % 8) ^ swz(row) of k-chunk w
+  // this lane's DMA sources at k = 0: row 8 i + l / 8 of the slab (i = 0..3) and of x
+  // (i < XR / 8; rows >= M re-read row M - 1), 16-byte chunk (l % 8) ^ swz(row) of a k-chunk
   const char* wsrc[4];
   const char* xsrc[XR / 8];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = 8 * i + (l >> 3);
-    wsrc[i] = W + (n0 + r) * ldw + 128 * w + (((l & 7) ^ GeoNK8::swz(r)) << 4);
+    wsrc[i] = W + (n0 + r) * ldw + (((l & 7) ^ GeoNK8::swz(r)) << 4);
     if (i < XR / 8)
-      xsrc[i] = X + (int64_t)(r < M ? r : M - 1) * ldx + 128 * w + (((l & 7) ^ GeoNK8::swz(r)) << 4);
+      xsrc[i] = X + (int64_t)(r < M ? r : M - 1) * ldx + (((l & 7) ^ GeoNK8::swz(r)) << 4);
   }
   // Workgroups start at different stages of K and wrap around (integer sums do not depend on
   // the order): at any moment they read different 512-byte columns of their rows, which spreads
   // the requests over the memory channels (19.4 -> 14.1 us per call at N = K = 8192).
   const int rot = (int)((blockIdx.x * 7u) % (unsigned)KTS);
-  auto issue = [&](int st, int slot) {
-    st = st < KTS ? st : KTS - 1;  // past the end: refetch the last stage into a dead slot
-    st += rot;
+  // first k of wave w's chunk of the s-th stage this workgroup visits, or -1 when that chunk
+  // lies past K (last stage of a K that is not a multiple of 512)
+  auto chunk_k = [&](int s) {
+    int st = s + rot;
     st = st < KTS ? st : st - KTS;
+    const int k = st * G::K_ELEMS + 128 * w;
+    return k < K ? k : -1;
+  };
+  auto issue = [&](int s, int slot) {
+    s = s < KTS ? s : KTS - 1;  // past the end: refetch the last stage into a dead slot
+    int k = chunk_k(s);
+    k = k >= 0 ? k : K - 128;   // a chunk past K: fetch the last valid one, never multiplied
     const uint32_t dst = lds_base + slot * G::STAGE_BYTES;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      dma16(wsrc[i] + (int64_t)st * G::K_ELEMS, dst + w * 4096 + (8 * i) * 128);
+    for (int i = 0; i < 4; ++i) dma16(wsrc[i] + k, dst + w * 4096 + (8 * i) * 128);
 #pragma unroll
     for (int i = 0; i < XR / 8; ++i)
-      dma16(xsrc[i] + (int64_t)st * G::K_ELEMS, dst + G::W_BYTES + w * (XR * 128) + (8 * i) * 128);
+      dma16(xsrc[i] + k, dst + G::W_BYTES + w * (XR * 128) + (8 * i) * 128);
   };
   auto wait_vmcnt = [](auto n_const) {
     constexpr int n = decltype(n_const)::value;
@@ -440,13 +449,16 @@ __global__ __launch_bounds__(256, 1) void skinny_nk8_kwaves_kernel(int M, int N,
     issue(s + DIST, dma_slot);
     const char* sw = lds + slot * G::STAGE_BYTES + w * 4096;
     const char* sx = lds + slot * G::STAGE_BYTES + G::W_BYTES + w * (XR * 128);
+    if (chunk_k(s) >= 0) {
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      // rows XR .. 31 of the padded x tile alias rows 0 .. XR - 1: never stored
-      const u32x4 xf =
-          *reinterpret_cast<const u32x4*>(sx + GeoNK8::off(l & (XR - 1), 2 * kk + (l >> 5)));
-      const u32x4 wf = *reinterpret_cast<const u32x4*>(sw + GeoNK8::off(l & 31, 2 * kk + (l >> 5)));
-      acc = Math::mfma(wf, xf, acc);
+      for (int kk = 0; kk < 4; ++kk) {
+        // rows XR .. 31 of the padded x tile alias rows 0 .. XR - 1: never stored
+        const u32x4 xf =
+            *reinterpret_cast<const u32x4*>(sx + GeoNK8::off(l & (XR - 1), 2 * kk + (l >> 5)));
+        const u32x4 wf =
+            *reinterpret_cast<const u32x4*>(sw + GeoNK8::off(l & 31, 2 * kk + (l >> 5)));
+        acc = Math::mfma(wf, xf, acc);
+      }
     }
     slot = slot + 1 == NS ? 0 : slot + 1;
     dma_slot = dma_slot + 1 == NS ? 0 : dma_slot + 1;
@@ -488,17 +500,20 @@ void launch_skinny_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, c
     attr_device = ctx->device;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN)), dim3(256), LDS_BYTES, ctx->stream, (int)M,
-                     (int)N, (int)(K / G::K_ELEMS), static_cast<const char*>(X), ldx_bytes,
+                     (int)N, (int)K, static_cast<const char*>(X), ldx_bytes,
                      static_cast<const char*>(W), ldw_bytes, epi);
 }
 
-// int8 N x K: the kernel above when it applies (a slab per compute unit, K in whole 512-k
-// stages), else the split-K kernel.  Returns true when the first one ran.
+// int8 N x K: the kernel above unless the weights are a few slabs of a very long K (then the
+// K ranges of the split-K kernel spread the stream over more compute units).  Measured at
+// M = 8, per call: 4096 x 8192 13.2 -> 10.1 us, 4096 x 4096 10.9 -> 7.2, 1024 x 8192 11.1 ->
+// 8.7, 128 x 8192 9.2 -> 7.2 (7.2 us is the floor of the test's launch path).
+// Returns true when the first one ran.
 template <typename Epi>
 bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
                        int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-  if (K % 512 == 0 && N % 32 == 0 && N / 32 >= cus) {
+  if (N / 32 >= cus / 4 || K <= 16384) {
     if (M <= 8)
       launch_skinny_kwaves<Epi, 8>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
     else if (M <= 16)

@@ -183,5 +183,5 @@ def test_random_cases_reach_every_family():
     for frag in ("f32_generic", "f32_mfma_small", "f32_mfma_256", "bf16_generic", "bf16_mfma_256",
                  "f16_mfma_256", "i8_generic", "i8_mfma_256x256x64_ring4_kn",
                  "i8_mfma_256x256x64_ring4_nk", "dequant", "bf16_skinny", "f16_skinny",
-                 "i8_skinny_32x128_ring7_nk", "i8_skinny_32x128_ring7_nk_dequant"):
+                 "i8_skinny_32x32_kwaves_nk", "i8_skinny_32x32_kwaves_nk_dequant"):
         assert any(frag in k for k in SEEN), (frag, sorted(SEEN))
