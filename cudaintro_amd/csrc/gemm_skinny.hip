@@ -513,7 +513,8 @@ template <typename Epi>
 bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
                        int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-  if (N / 32 >= cus / 4 || K <= 16384) {
+  // (N not a multiple of the split-K kernel's 128-column slabs: only this kernel takes it)
+  if (N / 32 >= cus / 4 || K <= 16384 || N % GeoNK8::BN) {
     if (M <= 8)
       launch_skinny_kwaves<Epi, 8>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
     else if (M <= 16)
@@ -538,6 +539,11 @@ bool skinny_shape_ok(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K, 
   return true;
 }
 
+// the shape conditions of the int8 kernel without split-K: 32-column slabs, 128-k chunks
+struct Slab32 {
+  static constexpr int BN = 32, K_ELEMS = 128;
+};
+
 }  // namespace
 
 bool launch_skinny_16(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_t K,
@@ -561,7 +567,7 @@ bool launch_skinny_i8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const
                       int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
                       int64_t ldc, const DequantArgs* dq) {
   if (!b_nk) return false;  // K x N int8 weights at M <= 32 go to the any-shape kernel
-  if (!skinny_shape_ok<GeoNK8>(ctx, M, N, K, 1, A, lda, B, ldb)) return false;
+  if (!skinny_shape_ok<Slab32>(ctx, M, N, K, 1, A, lda, B, ldb)) return false;
   if (!dq) {
     if (ldc % 4 || ((uintptr_t)C & 15)) return false;
     const bool kw = launch_skinny_nk8(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32x4{C, ldc});

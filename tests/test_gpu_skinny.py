@@ -97,6 +97,7 @@ def test_skinny_int8_nk(handle, torch_gpu, oracle, rng, M, N, K, out_type):
 
 @pytest.mark.parametrize("M", [1, 5, 8, 9, 16, 17, 32])
 @pytest.mark.parametrize("N,K", [(8192, 512), (8192 + 128, 1536), (8192, 4096 + 128), (128, 128), (256, 640),
+                                 (32, 256), (8192 + 96, 1024), (160, 16384 + 640),
                                  (2048, 16384 + 384), (256, 16384 + 512), (1024, 32768 + 128)])
 def test_skinny_int8_without_split_k(handle, torch_gpu, oracle, rng, M, N, K):
     """The kernel that splits K over the waves of a workgroup instead of over workgroups, with
@@ -109,7 +110,7 @@ def test_skinny_int8_without_split_k(handle, torch_gpu, oracle, rng, M, N, K):
     W = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
     acc_ref = oracle.gemm_i8_i32(X, W, b_is_nk=True)
     xd, wd = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda()
-    expect_kw = N >= 2048 or K <= 16384
+    expect_kw = N >= 2048 or K <= 16384 or N % 128 != 0
     out = torch.full((M + 2, N + 4), -9, dtype=torch.int32, device="cuda")
     for _ in range(2):
         handle.gemm_i8_i32(xd, wd, ci.B_NK, out=out[:M, :N])
