@@ -110,7 +110,7 @@ typedef enum cigemmAlgo {
   CIGEMM_ALGO_DEFAULT = -1,
   CIGEMM_ALGO_GENERIC = 0, /* any-shape scalar kernel (fp32: bit-exact with the CPU loop) */
   CIGEMM_ALGO_TILE = 1,    /* LDS-tiled MFMA kernel, 256-column tiles */
-  CIGEMM_ALGO_SKINNY = 2,  /* M <= 32 split-K streaming kernel (16-bit K x N, int8 N x K) */
+  CIGEMM_ALGO_SKINNY = 2,  /* M <= 32 weight-streaming kernels (16-bit K x N, int8 N x K) */
   CIGEMM_ALGO_SMALL = 3    /* fp32 32x32 tile per workgroup, k split over the waves */
 } cigemmAlgo_t;
 CIGEMM_API cigemmStatus_t cigemmSetAlgo(cigemmHandle_t handle, cigemmAlgo_t algo);
