@@ -168,6 +168,26 @@ def cpu_baseline_16bit(Ab, Bb, kind, target_seconds=12.0):
                       f"fp32 i-j-k triple loop, {dt:.1f} s"}
 
 
+def cpu_rows_baseline(run_rows, M, ops_per_row, unit, what, target_seconds=3.0):
+    """Times `run_rows(r)` (the CPU port on the first r rows of the problem; cost is exactly
+    linear in rows) on a bounded slice: a probe of a few rows, then as many rows as fit
+    `target_seconds`.  Returns the per_config[*].cpu_baseline object and run_rows' last result."""
+    import oracle
+    threads = oracle.num_threads()
+    rows = min(M, max(threads, 8))
+    t0 = time.perf_counter()
+    run_rows(rows)
+    dt = time.perf_counter() - t0
+    rows2 = min(M, max(rows, int(rows * target_seconds / max(dt, 1e-4))))
+    if rows2 >= threads:
+        rows2 -= rows2 % threads
+    t0 = time.perf_counter()
+    res = run_rows(rows2)
+    dt = time.perf_counter() - t0
+    return {"value": ops_per_row * rows2 / dt / 1e12, "unit": unit, "cores": min(threads, rows2),
+            "kind": "port", "sample": f"first {rows2} of {M} rows of the same problem, {what}, {dt:.2f} s"}, res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -178,9 +198,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--reference-seconds", type=float, default=3.0,
-                    help="time budget per precision of the reference's own protocol (its driver "
-                         "uses 10; 0 skips that leg)")
+    ap.add_argument("--reference-seconds", type=float, default=10.0,
+                    help="time budget per precision of the reference's own protocol (10, as in "
+                         "quantization/GEMM_bf16.cu:63; 0 skips that leg)")
     ap.add_argument("--size", type=int, default=8192, help="headline M=N=K (default 8192)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy a few times (reference point for "
@@ -228,9 +248,30 @@ def main():
                 "avg_kernel_ms": ev / args.steps * 1e3}
     roofline["median_kernel_ms"] = median_call_ms(torch, lambda: handle.gemm_bf16(A, B, out=C),
                                                   max(50, args.steps))
+    # HBM-side bytes per launch and the counter decomposition of the same kernel are not
+    # measurable from inside this process: they come from the rocprofv3 --pmc runs of this
+    # same command summarised in profiles/ (the file says which runs).
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file):
-        roofline["traffic"] = json.load(open(traffic_file)).get(f"bf16_{n}")
+        prof = json.load(open(traffic_file))
+        roofline["traffic"] = prof.get(f"bf16_{n}")
+        roofline["traffic_source"] = "profiles/hbm_traffic.json"
+        for key in ("mfma_busy", "clock_ghz"):
+            if f"bf16_{n}_{key}" in prof:
+                roofline[key] = prof[f"bf16_{n}_{key}"]
+                roofline[key + "_source"] = "profiles/hbm_traffic.json"
+    # What a register-resident loop of the same matrix instruction sustains in this run on
+    # random operand bits, with no memory traffic at all: the chip is power limited on such
+    # data, so this, not the datasheet peak, is the ceiling a kernel can approach.
+    ops_box = [0]
+
+    def fn_probe():
+        ops_box[0] = handle.probe_mfma("bf16", True, 20000)
+    _, e_probe = time_calls(torch, fn_probe, 20, 10)
+    roofline["sustained_peak"] = ops_box[0] * 20 / e_probe / 1e12
+    roofline["sustained_peak_what"] = ("register-resident v_mfma_f32_32x32x16_bf16 loop, random "
+                                       "operand bits, one wave per SIMD, same run")
+    roofline["frac_of_sustained"] = achieved / roofline["sustained_peak"]
 
     cpu = None
     if not args.no_cpu:
@@ -272,6 +313,24 @@ def main():
             t = wl.gemm_ops(M, N, K) * args.steps / e / 1e12
             per_config[name] = {"tops": t, "frac_of_peak": t / PEAK_INT8_TOPS, "peak": PEAK_INT8_TOPS,
                                 "ms": e / args.steps * 1e3, "kernel": handle.last_kernel}
+            if not args.no_cpu:
+                # the int8 -> int32 twin of the reference's CPU loop on a slice of rows, timed;
+                # the same rows of the GPU result are compared with it (bit-exact or not)
+                import oracle
+                nk = lay == ci.B_NK
+                base, acc_ref = cpu_rows_baseline(lambda r: oracle.gemm_i8_i32(Aq[:r], Bq, b_is_nk=nk), M,
+                                                  2.0 * N * K, "TOP/s", "int8 x int8 -> int32 loop")
+                r = acc_ref.shape[0]
+                if dequant:
+                    bf = out_t == ci.OUT_BF16
+                    want = oracle.dequant(acc_ref, sa[:r] if sa.size > 1 else sa, sb,
+                                          out_dtype="bf16" if bf else "f32",
+                                          sa_per_row=sa.size > 1, sb_per_col=sb.size > 1)
+                    got = out[:r].view(torch.int16).cpu().numpy().view(np.uint16) if bf else out[:r].cpu().numpy()
+                else:
+                    want, got = acc_ref, out[:r].cpu().numpy()
+                base["gpu_rows_bit_exact"] = bool(np.array_equal(got, want))
+                per_config[name]["cpu_baseline"] = base
 
         def mk_square(sz, seed):
             def f():
@@ -367,6 +426,18 @@ def main():
             per_config[f"skinny_bf16_M{M}"] = {"gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS,
                                                "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
                                                "bytes": nbytes, "kernel": handle.last_kernel}
+            if not args.no_cpu:
+                # the reference's fp32 i-j-k loop on the widened inputs, on the rows that fit
+                import oracle
+                xf, wf = wl.widen_16bit(xb, "bf16"), wl.widen_16bit(wb, "bf16")
+                base, cpu_rows = cpu_rows_baseline(lambda r: oracle.gemm_f32_ijk(xf, wf, 0, r)[:r], M,
+                                                   2.0 * 8192 * 8192, "TFLOP/s", "fp32 i-j-k triple loop",
+                                                   target_seconds=2.0)
+                r = cpu_rows.shape[0]
+                got = wl.bf16_bits_to_f32(y[:r].view(torch.int16).cpu().numpy().view(np.uint16))
+                base["gpu_rows_max_abs_diff"] = float(np.abs(got - cpu_rows).max())
+                base["cpu_rows_rms"] = float(np.sqrt(np.mean(cpu_rows.astype(np.float64) ** 2)))
+                per_config[f"skinny_bf16_M{M}"]["cpu_baseline"] = base
             del ws
             xq, sx, wq, sw = wl.skinny_int8(M, 8192, 8192, seed=4)
             xd, sxd, swd = torch.from_numpy(xq).cuda(), torch.from_numpy(sx).cuda(), torch.from_numpy(sw).cuda()
@@ -382,6 +453,17 @@ def main():
             per_config[f"skinny_int8_M{M}"] = {"gbs": gbs, "frac_of_peak": gbs / PEAK_HBM_GBS,
                                                "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
                                                "bytes": nbytes, "kernel": handle.last_kernel}
+            if not args.no_cpu:
+                import oracle
+                base, acc_ref = cpu_rows_baseline(lambda r: oracle.gemm_i8_i32(xq[:r], wq, b_is_nk=True), M,
+                                                  2.0 * 8192 * 8192, "TOP/s", "int8 x int8 -> int32 loop",
+                                                  target_seconds=1.0)
+                r = acc_ref.shape[0]
+                want = oracle.dequant(acc_ref, sx[:r] if M > 1 else sx, sw, out_dtype="bf16",
+                                      sa_per_row=M > 1, sb_per_col=True)
+                base["gpu_rows_bit_exact"] = bool(np.array_equal(
+                    yo[:r].view(torch.int16).cpu().numpy().view(np.uint16), want))
+                per_config[f"skinny_int8_M{M}"]["cpu_baseline"] = base
             del wqs
         # small-batch shapes between the decode and the square configurations: few output
         # tiles and a long K, run as split-K (weights still dominate the traffic)

@@ -28,9 +28,11 @@ class Status(enum.IntEnum):
     ALLOC_FAILED = 3
     INVALID_VALUE = 7
     ARCH_MISMATCH = 8
+    MAPPING_ERROR = 11
     EXECUTION_FAILED = 13
     INTERNAL_ERROR = 14
     NOT_SUPPORTED = 15
+    LICENSE_ERROR = 16
 
 
 class CigemmError(RuntimeError):
@@ -111,6 +113,7 @@ def load_library():
 def _torch():
     import torch
     return torch
+
 
 
 class Handle:

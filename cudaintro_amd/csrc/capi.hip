@@ -20,11 +20,48 @@ cigemmStatus_t fail(cigemmContext* ctx, cigemmStatus_t st, const char* fmt, ...)
 }
 
 cigemmStatus_t check_launch(cigemmContext* ctx, const char* what) {
+  if (ctx && ctx->pending_error[0]) {
+    char msg[sizeof(ctx->pending_error)];
+    memcpy(msg, ctx->pending_error, sizeof(msg));
+    ctx->pending_error[0] = '\0';
+    (void)hipGetLastError();
+    return fail(ctx, CIGEMM_STATUS_INTERNAL_ERROR, "%s: %s", what, msg);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess)
     return fail(ctx, CIGEMM_STATUS_EXECUTION_FAILED, "%s: HIP error: %s", what,
                 hipGetErrorString(e));
   return CIGEMM_STATUS_SUCCESS;
+}
+
+void set_tile_kernel_name(cigemmContext* ctx, const char* dtype, int k_elems, const char* suffix,
+                          bool splitk) {
+  char rows[24], waves[24];
+  if (ctx->first_tile_rows) {
+    snprintf(rows, sizeof(rows), "%d+%d", ctx->first_tile_rows, ctx->last_tile_rows);
+    snprintf(waves, sizeof(waves), "w%d+w%d", ctx->first_waves, ctx->last_waves);
+  } else {
+    snprintf(rows, sizeof(rows), "%d", ctx->last_tile_rows);
+    snprintf(waves, sizeof(waves), "w%d", ctx->last_waves);
+  }
+  snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_mfma_%sx256x%d_%s_ring4%s%s", dtype,
+           rows, k_elems, waves, suffix, splitk ? "_splitk" : "");
+  ctx->last_kernel = ctx->kernel_name;
+}
+
+void ensure_dynamic_lds(cigemmContext* ctx, const void* kernel, int bytes,
+                        std::atomic<uint64_t>& done) {
+  const uint64_t bit = 1ull << (ctx->device & 63);
+  if (done.load(std::memory_order_acquire) & bit) return;
+  const hipError_t e =
+      hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    snprintf(ctx->pending_error, sizeof(ctx->pending_error),
+             "the device refused %d bytes of LDS per workgroup (%s)", bytes, hipGetErrorString(e));
+    return;
+  }
+  done.fetch_or(bit, std::memory_order_release);
 }
 
 namespace {
@@ -37,6 +74,9 @@ cigemmStatus_t check_gemm_args(cigemmHandle_t h, const char* name, int64_t M, in
                                int64_t ldb, int64_t b_cols, const void* C, int64_t ldc) {
   h->last_tile_rows = 0;  // set again by the tile kernel's launcher
   h->last_k_splits = 0;
+  h->last_waves = 0;
+  h->first_tile_rows = 0;
+  h->first_waves = 0;
   if (M < 0 || N < 0 || K < 0)
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: negative dimension (M=%lld N=%lld K=%lld)",
                 name, (long long)M, (long long)N, (long long)K);
@@ -92,6 +132,11 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->last_kernel = "";
   ctx->last_tile_rows = 0;
   ctx->last_k_splits = 0;
+  ctx->last_waves = 0;
+  ctx->first_tile_rows = 0;
+  ctx->first_waves = 0;
+  ctx->kernel_name[0] = '\0';
+  ctx->pending_error[0] = '\0';
   ctx->algo = CIGEMM_ALGO_DEFAULT;
   ctx->last_error[0] = '\0';
   ctx->ws_partial_bytes = (size_t)64 << 20;
@@ -137,9 +182,11 @@ const char* cigemmGetStatusString(cigemmStatus_t status) {
     case CIGEMM_STATUS_ALLOC_FAILED: return "CIGEMM_STATUS_ALLOC_FAILED";
     case CIGEMM_STATUS_INVALID_VALUE: return "CIGEMM_STATUS_INVALID_VALUE";
     case CIGEMM_STATUS_ARCH_MISMATCH: return "CIGEMM_STATUS_ARCH_MISMATCH";
+    case CIGEMM_STATUS_MAPPING_ERROR: return "CIGEMM_STATUS_MAPPING_ERROR";
     case CIGEMM_STATUS_EXECUTION_FAILED: return "CIGEMM_STATUS_EXECUTION_FAILED";
     case CIGEMM_STATUS_INTERNAL_ERROR: return "CIGEMM_STATUS_INTERNAL_ERROR";
     case CIGEMM_STATUS_NOT_SUPPORTED: return "CIGEMM_STATUS_NOT_SUPPORTED";
+    case CIGEMM_STATUS_LICENSE_ERROR: return "CIGEMM_STATUS_LICENSE_ERROR";
     default: return "CIGEMM_STATUS_UNKNOWN";
   }
 }

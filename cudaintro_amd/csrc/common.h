@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -18,6 +19,13 @@ struct cigemmContext {
   const char* last_kernel;
   int last_tile_rows;  // rows of the output tile of the last tile-kernel launch, 0 otherwise
   int last_k_splits;   // K ranges of that launch
+  int last_waves;      // wavefronts per workgroup of that launch
+  int first_tile_rows; // when the call took two launches: rows and waves of the first, else 0
+  int first_waves;
+  char kernel_name[96];  // storage for names composed per call (last_kernel may point here)
+  // A failure recorded while a launch was being prepared (a refused kernel attribute), reported
+  // by check_launch as CIGEMM_STATUS_INTERNAL_ERROR; empty when there is none.
+  char pending_error[160];
   int algo;  // cigemmAlgo_t; -1 = choose by shape
   // Device scratch of the split-K kernels, allocated once at create: `ws_partial_bytes` of
   // partial sums followed by `ws_counter_bytes` of arrival counters (zero between calls).
@@ -35,6 +43,16 @@ namespace cig {
 cigemmStatus_t fail(cigemmContext* ctx, cigemmStatus_t st, const char* fmt, ...)
     __attribute__((format(printf, 3, 4)));
 cigemmStatus_t check_launch(cigemmContext* ctx, const char* what);
+// Name of a tile-kernel call from what the launcher recorded on the context, e.g.
+// "i8_mfma_192x256x64_w4_ring4_nk_dequant" (tile rows x 256 columns x k elements per stage,
+// waves per workgroup), "256+192" / "w4+w4" when two launches covered the columns.
+void set_tile_kernel_name(cigemmContext* ctx, const char* dtype, int k_elems, const char* suffix,
+                          bool splitk);
+// Raises the dynamic-LDS limit of `kernel` to `bytes` once per device and template instance
+// (`done` = that instance's bit mask of devices already set).  A refusal is recorded on the
+// context and reported by check_launch.
+void ensure_dynamic_lds(cigemmContext* ctx, const void* kernel, int bytes,
+                        std::atomic<uint64_t>& done);
 
 // ---- vector types ---------------------------------------------------------------------
 typedef float f32x4 __attribute__((ext_vector_type(4)));

@@ -15,11 +15,11 @@ bool launch_16b_mfma(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_
   if (bf16) {
     const bool split = tile::launch_tile<tile::MathBF16, tile::B_KN16>(
         ctx, M, N, K * 2, A, lda * 2, B, ldb * 2, EpiStore16x4<BF16>{C, ldc});
-    ctx->last_kernel = split ? "bf16_mfma_256x256x32_ring4_splitk" : "bf16_mfma_256x256x32_ring4";
+    set_tile_kernel_name(ctx, "bf16", 32, "", split);
   } else {
     const bool split = tile::launch_tile<tile::MathF16, tile::B_KN16>(
         ctx, M, N, K * 2, A, lda * 2, B, ldb * 2, EpiStore16x4<F16>{C, ldc});
-    ctx->last_kernel = split ? "f16_mfma_256x256x32_ring4_splitk" : "f16_mfma_256x256x32_ring4";
+    set_tile_kernel_name(ctx, "f16", 32, "", split);
   }
   return true;
 }

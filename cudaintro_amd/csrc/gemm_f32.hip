@@ -49,7 +49,7 @@ bool launch_f32_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const 
   if (!ba) {
     const bool split = tile::launch_tile<tile::MathF32, tile::B_KN32>(
         ctx, M, N, K * 4, A, lda * 4, B, ldb * 4, EpiStoreF32x4{C, ldc});
-    ctx->last_kernel = split ? "f32_mfma_256x256x16_ring4_splitk" : "f32_mfma_256x256x16_ring4";
+    set_tile_kernel_name(ctx, "f32", 16, "", split);
     return true;
   }
   bool split = false;
@@ -62,8 +62,7 @@ bool launch_f32_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const 
     if (ba->relu) CIG_BA(false, true); else CIG_BA(false, false);
   }
 #undef CIG_BA
-  ctx->last_kernel = split ? "f32_mfma_256x256x16_ring4_bias_act_splitk"
-                           : "f32_mfma_256x256x16_ring4_bias_act";
+  set_tile_kernel_name(ctx, "f32", 16, "_bias_act", split);
   return true;
 }
 

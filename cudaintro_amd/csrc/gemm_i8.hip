@@ -46,12 +46,8 @@ bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const i
   }
   const bool split = b_nk ? launch_layout<tile::B_NK>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq)
                           : launch_layout<tile::B_KN8>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
-  static const char* const names[2][2][2] = {
-      {{"i8_mfma_256x256x64_ring4_kn", "i8_mfma_256x256x64_ring4_kn_splitk"},
-       {"i8_mfma_256x256x64_ring4_nk", "i8_mfma_256x256x64_ring4_nk_splitk"}},
-      {{"i8_mfma_256x256x64_ring4_kn_dequant", "i8_mfma_256x256x64_ring4_kn_dequant_splitk"},
-       {"i8_mfma_256x256x64_ring4_nk_dequant", "i8_mfma_256x256x64_ring4_nk_dequant_splitk"}}};
-  ctx->last_kernel = names[dq ? 1 : 0][b_nk ? 1 : 0][split ? 1 : 0];
+  set_tile_kernel_name(ctx, "i8", 64, dq ? (b_nk ? "_nk_dequant" : "_kn_dequant") : (b_nk ? "_nk" : "_kn"),
+                       split);
   return true;
 }
 

@@ -329,12 +329,8 @@ void launch_skinny_n(cigemmContext* ctx, int64_t M, int64_t N, int64_t kts, cons
                      int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
   constexpr int LDS_BYTES = Geo::NSTAGES * Geo::STAGE_BYTES;
   auto kern = skinny_kernel<Geo, Epi, SPLITS>;
-  static int attr_device = -1;
-  if (attr_device != ctx->device) {
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              LDS_BYTES);
-    attr_device = ctx->device;
-  }
+  static std::atomic<uint64_t> lds_set{0};
+  ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set);
   const unsigned grid = (unsigned)((N / Geo::BN) * SPLITS);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS_BYTES, ctx->stream, (int)M, (int)N,
                      (int)(kts / SPLITS), static_cast<const char*>(X), ldx_bytes,
@@ -493,12 +489,8 @@ void launch_skinny_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, c
   constexpr int LDS_BYTES = G::NSTAGES * G::STAGE_BYTES;
   static_assert(LDS_BYTES <= 160 * 1024, "ring must fit the LDS");
   auto kern = skinny_nk8_kwaves_kernel<Epi, XR>;
-  static int attr_device = -1;
-  if (attr_device != ctx->device) {
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              LDS_BYTES);
-    attr_device = ctx->device;
-  }
+  static std::atomic<uint64_t> lds_set{0};
+  ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set);
   hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN)), dim3(256), LDS_BYTES, ctx->stream, (int)M,
                      (int)N, (int)K, static_cast<const char*>(X), ldx_bytes,
                      static_cast<const char*>(W), ldw_bytes, epi);

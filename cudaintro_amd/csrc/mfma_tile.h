@@ -773,15 +773,12 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
   constexpr int STAGING_BYTES = 2 * WM * 32 * (128 * Epi::OUT_BYTES + 16);   // epilogue, per wave
   constexpr int LDS_BYTES = RING_BYTES > STAGING_BYTES ? RING_BYTES : STAGING_BYTES;
   auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, MT, Epi, WM>;
-  static int attr_device = -1;  // one per template instance
-  if (attr_device != ctx->device) {
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              LDS_BYTES);
-    attr_device = ctx->device;
-  }
+  static std::atomic<uint64_t> lds_set{0};  // one per template instance
+  ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set);
   const int tiles_m = (int)((M + TILE_M - 1) / TILE_M), tiles_n = (int)((N + BN - 1) / BN);
   ctx->last_tile_rows = TILE_M;
   ctx->last_k_splits = splits;
+  ctx->last_waves = 2 * WM;
   const int64_t kts = K_bytes / KB / splits;  // stages per K range
   const int64_t a_step = kts * KB;
   const int64_t b_step = BMODE == B_NK ? kts * KB : kts * (KB / Math::ELEM_BYTES) * ldb_bytes;
@@ -1002,10 +999,13 @@ bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
         const int mt2 = best_mt(M, n2, cus, &rest);
         if (tile_plan_cost(M, n1, 4, cus) + rest < single * 0.97) {
           launch_tile_256<Math, BMODE>(ctx, M, n1, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+          const int rows1 = ctx->last_tile_rows, waves1 = ctx->last_waves;
           const char* B2 = static_cast<const char*>(B) +
                            (BMODE == B_NK ? n1 * ldb_bytes : n1 * Math::ELEM_BYTES);
           launch_tile_any_mt<Math, BMODE>(ctx, mt2, M, n2, K_bytes, A, lda_bytes, B2, ldb_bytes,
                                           epi.shift_cols(n1));
+          ctx->first_tile_rows = rows1;
+          ctx->first_waves = waves1;
           return false;
         }
       }

@@ -40,9 +40,11 @@ typedef enum cigemmStatus {
   CIGEMM_STATUS_ALLOC_FAILED = 3,
   CIGEMM_STATUS_INVALID_VALUE = 7,    /* null pointer, negative size, ld too small ... */
   CIGEMM_STATUS_ARCH_MISMATCH = 8,    /* device is not gfx950                          */
+  CIGEMM_STATUS_MAPPING_ERROR = 11,   /* kept for the reference's table; never returned */
   CIGEMM_STATUS_EXECUTION_FAILED = 13,/* HIP reported a launch / runtime error         */
   CIGEMM_STATUS_INTERNAL_ERROR = 14,
-  CIGEMM_STATUS_NOT_SUPPORTED = 15    /* valid arguments, combination not implemented  */
+  CIGEMM_STATUS_NOT_SUPPORTED = 15,   /* valid arguments, combination not implemented  */
+  CIGEMM_STATUS_LICENSE_ERROR = 16    /* kept for the reference's table; never returned */
 } cigemmStatus_t;
 
 /* Opaque library context (device, stream).  Takes the place of cublasHandle_t. */
@@ -90,8 +92,12 @@ CIGEMM_API const char* cigemmGetLastErrorString(cigemmHandle_t handle);
 /* Library version, major*10000 + minor*100 + patch. */
 CIGEMM_API int cigemmGetVersion(void);
 
-/* Name of the kernel family the last successful GEMM call on this handle dispatched to
- * (for tests and profiles), e.g. "bf16_mfma_256x256x32_ring4". */
+/* Name of the kernel the last successful GEMM call on this handle dispatched to (for tests and
+ * profiles).  The LDS-tiled matrix-core kernel reports its real plan:
+ * "<type>_mfma_<tile rows>x256x<k per stage>_w<waves per workgroup>_ring4[_kn|_nk][_dequant]
+ * [_bias_act][_splitk]", e.g. "bf16_mfma_256x256x32_w4_ring4", "i8_mfma_256+192x256x64_w8+w4_
+ * ring4_nk_dequant" when two launches of different tile heights covered the columns.  Valid
+ * until the next GEMM call on the handle. */
 CIGEMM_API const char* cigemmGetLastKernelName(cigemmHandle_t handle);
 
 /* Plan of the last successful GEMM call on this handle, for tests and profiles: rows of the

@@ -59,6 +59,12 @@ def test_status_strings_and_null_handle():
     assert lib.cigemmGetStatusString(0) == b"CIGEMM_STATUS_SUCCESS"
     assert lib.cigemmGetStatusString(7) == b"CIGEMM_STATUS_INVALID_VALUE"
     assert lib.cigemmGetStatusString(99) == b"CIGEMM_STATUS_UNKNOWN"
+    # every name the reference's table prints (quantization/gemm_common.h:10-35) has a counterpart
+    for code, name in {0: "SUCCESS", 1: "NOT_INITIALIZED", 3: "ALLOC_FAILED", 7: "INVALID_VALUE",
+                       8: "ARCH_MISMATCH", 11: "MAPPING_ERROR", 13: "EXECUTION_FAILED",
+                       14: "INTERNAL_ERROR", 15: "NOT_SUPPORTED", 16: "LICENSE_ERROR"}.items():
+        assert lib.cigemmGetStatusString(code) == b"CIGEMM_STATUS_" + name.encode()
+        assert cigemm.Status(code).name == name
     assert lib.cigemmGetVersion() >= 100
     # null handle: status code, never a crash
     assert lib.cigemmDestroy(None) == cigemm.Status.NOT_INITIALIZED

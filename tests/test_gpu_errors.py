@@ -92,7 +92,7 @@ def test_kernel_family_selection(torch_gpu):
             h.gemm_i8_i32(a8, a8)
     torch.cuda.synchronize()
     assert (out.cpu().numpy() == 5.0).all()
-    for algo, frag in ((ci.ALGO_GENERIC, "generic"), (ci.ALGO_TILE, "mfma_256"), (ci.ALGO_DEFAULT, "mfma")):
+    for algo, frag in ((ci.ALGO_GENERIC, "generic"), (ci.ALGO_TILE, "x256x"), (ci.ALGO_DEFAULT, "mfma")):
         h.set_algo(algo)
         c = h.gemm_bf16(a16, a16)
         assert frag in h.last_kernel

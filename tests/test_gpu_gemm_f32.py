@@ -151,7 +151,7 @@ def test_tile_kernel_ragged_shapes(handle, torch_gpu, oracle, rng, shape):
     """Any M, N a multiple of 4, K a multiple of 16 go through the MFMA tile kernel with
     clamped loads and masked stores; guard rows/columns of the output stay untouched."""
     name = ragged_check(handle, torch_gpu, oracle, rng, ci.ALGO_TILE, shape)
-    assert "mfma_256" in name, name
+    assert "x256x16_w" in name, name
 
 
 @pytest.mark.parametrize("shape", [(33, 4, 16), (100, 260, 48), (257, 1028, 64), (1000, 12, 512),
@@ -236,9 +236,9 @@ def test_default_choice_by_shape(handle, torch_gpu):
     assert "small" in kernel_for(512, 512, 512)
     assert "small" in kernel_for(1024, 1024, 1024)
     assert "small_16x16" in kernel_for(20000, 10, 512)
-    assert "mfma_256" in kernel_for(2048, 2048, 2048)
-    assert "mfma_256" in kernel_for(4096, 4096, 64)
-    assert "mfma_256" in kernel_for(20000, 512, 784)
+    assert "x256x16_w" in kernel_for(2048, 2048, 2048)
+    assert "x256x16_w" in kernel_for(4096, 4096, 64)
+    assert "x256x16_w" in kernel_for(20000, 512, 784)
     assert kernel_for(512, 512, 4096).endswith("_splitk")      # long K: tile kernel, K split
     assert kernel_for(256, 1024, 8192).endswith("_splitk")
     assert "generic" in kernel_for(77, 91, 300)

@@ -32,7 +32,7 @@ def test_mnist_hidden_layer(handle, torch_gpu, oracle, rng):
     X = rng.uniform(0, 1, size=(20000, 784)).astype(np.float32)
     W = (rng.normal(size=(784, 512)) * np.sqrt(2.0 / 784)).astype(np.float32)
     b = rng.normal(size=512).astype(np.float32) * 0.1
-    out = check(handle, torch_gpu, oracle, X, W, b, True, expect="mfma_256")
+    out = check(handle, torch_gpu, oracle, X, W, b, True, expect="x256x16_w")
     assert (out == 0).mean() > 0.1      # ReLU actually clips something
 
 
@@ -65,7 +65,7 @@ def test_each_kernel_family(handle, torch_gpu, oracle, rng, algo, shape, relu, w
     X = rng.uniform(-1, 1, size=(M, K)).astype(np.float32)
     W = rng.uniform(-1, 1, size=(K, N)).astype(np.float32)
     b = rng.uniform(-1, 1, size=N).astype(np.float32) if with_bias else None
-    expect = {ci.ALGO_GENERIC: "generic", ci.ALGO_TILE: "mfma_256", ci.ALGO_SMALL: "small"}[algo]
+    expect = {ci.ALGO_GENERIC: "generic", ci.ALGO_TILE: "x256x16_w", ci.ALGO_SMALL: "small"}[algo]
     check(handle, torch_gpu, oracle, X, W, b, relu, expect=expect, algo=algo)
 
 

@@ -180,8 +180,8 @@ def test_random_int8(handle, torch_gpu, oracle, layout, case):
 
 def test_random_cases_reach_every_family():
     """The draws above are only worth something if they exercise the fast paths too."""
-    for frag in ("f32_generic", "f32_mfma_small", "f32_mfma_256", "bf16_generic", "bf16_mfma_256",
-                 "f16_mfma_256", "i8_generic", "i8_mfma_256x256x64_ring4_kn",
-                 "i8_mfma_256x256x64_ring4_nk", "dequant", "bf16_skinny", "f16_skinny",
+    for frag in ("f32_generic", "f32_mfma_small", "x256x16_w", "bf16_generic", "bf16_mfma_",
+                 "f16_mfma_", "i8_generic", "_ring4_kn", "_ring4_nk", "dequant", "bf16_skinny",
+                 "f16_skinny",
                  "i8_skinny_32x32_kwaves_nk", "i8_skinny_32x32_kwaves_nk_dequant"):
         assert any(frag in k for k in SEEN), (frag, sorted(SEEN))

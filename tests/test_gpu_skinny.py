@@ -150,3 +150,27 @@ def test_config_skinny_decode(handle, torch_gpu, oracle):
         np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
         np.testing.assert_array_equal(bits(torch, out),
                                       oracle.dequant(acc_ref, sx, sw, out_dtype="bf16", sa_per_row=M > 1))
+
+
+@pytest.mark.parametrize("shape", [(5, 1024, 2048), (8, 8192, 8192)])
+def test_skinny_workspace_reuse_with_alternating_inputs(handle, torch_gpu, oracle, rng, shape):
+    """The split-K kernel's partials and arrival counters live in the handle's workspace: two
+    different problems of one shape called X, Y, X, Y on one handle, each checked against the
+    oracle (exact-arithmetic inputs: any summation order gives the same bits).  A stale partial
+    or a counter that did not return to zero would show as the other problem's values."""
+    torch = torch_gpu
+    M, N, K = shape
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    probs = []
+    for _ in range(2):
+        X, W = rng.choice(vals, size=(M, K)), rng.choice(vals, size=(K, N))
+        # keep |sums| small enough that fp32 partial sums stay exact at K = 8192
+        W[rng.random(size=W.shape) < 0.5] = 0
+        probs.append((to_dev(torch, oracle.f32_to_bf16(X), "bf16"), to_dev(torch, oracle.f32_to_bf16(W), "bf16"),
+                      oracle.f32_to_bf16(oracle.gemm_f32(X, W))))
+    assert not np.array_equal(probs[0][2], probs[1][2])
+    for i in range(6):
+        x, w, want = probs[i & 1]
+        y = handle.gemm_bf16(x, w)
+        assert "skinny" in handle.last_kernel, handle.last_kernel
+        np.testing.assert_array_equal(bits(torch, y), want, err_msg=f"call {i}")

@@ -44,3 +44,24 @@ def test_fill_kernels_division_free_forms_are_exact(tmp_path):
     out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout + out.stderr
     assert "exact arithmetic OK" in out.stdout
+
+
+def test_gemm_suite_exits_with_the_reference_message_without_a_device():
+    """The driver keeps the reference's fail-fast behaviour (quantization/gemm_common.h:47-55):
+    a failing library call prints "cigemm error: <status> at <file>:<line>" to stderr and exits
+    with status 1.  Without a GPU the first such call is cigemmCreate."""
+    import re
+
+    import pytest
+    import torch
+
+    import cudaintro_amd
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present: cigemmCreate succeeds")
+    exe = cudaintro_amd.suite_path()
+    assert os.path.exists(exe), "gemm_suite is not built"
+    out = subprocess.run([exe, "--seconds", "0.01", "--size", "256"], capture_output=True, text=True,
+                         timeout=120)
+    assert out.returncode == 1, (out.returncode, out.stderr)
+    assert re.search(r"cigemm error: CIGEMM_STATUS_\w+ at \S*main\.cpp:\d+\s*$", out.stderr), out.stderr
+    assert "Running" not in out.stdout
