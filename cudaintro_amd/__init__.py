@@ -24,6 +24,7 @@ from .cigemm import (  # noqa: F401
     Handle,
     Status,
     build_library,
+    gemm_bf16_static,
     library_path,
     load_library,
     suite_path,

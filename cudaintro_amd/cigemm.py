@@ -80,6 +80,8 @@ SIGNATURES = {
     "cigemm_gemm_f32": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "cigemm_gemm_f16": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "cigemm_gemm_bf16": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
+    "cigemm_gemm_bf16_static": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64,
+                                      C.c_char_p, C.c_size_t]),
     "cigemm_gemm_i8_i32": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _ci, _vp, _i64]),
     "cigemm_gemm_i8_dequant": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _ci, _vp, _ci,
                                      _vp, _ci, _vp, _ci, _i64, _vp, _i64]),
@@ -114,6 +116,26 @@ def _torch():
     import torch
     return torch
 
+
+def gemm_bf16_static(A, B, out=None, stream=None):
+    """``cigemm_gemm_bf16_static``: the decode-shape bf16 GEMM without a handle and without any
+    allocation inside the library (``out`` is allocated here, by torch, when not given)."""
+    torch = _torch()
+    lib = load_library()
+    assert A.dtype == torch.bfloat16 and B.dtype == torch.bfloat16
+    M, K = A.shape
+    K2, N = B.shape
+    assert K == K2
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
+    s = torch.cuda.current_stream() if stream is None else stream
+    err = C.create_string_buffer(256)
+    st = lib.cigemm_gemm_bf16_static(_vp(s.cuda_stream), M, N, K, A.data_ptr(), Handle._ld(A),
+                                     B.data_ptr(), Handle._ld(B), out.data_ptr(), Handle._ld(out),
+                                     err, len(err))
+    if st != 0:
+        raise CigemmError(st, err.value.decode(), "cigemm_gemm_bf16_static")
+    return out
 
 
 class Handle:

@@ -20,6 +20,10 @@
 //
 // int8 weights with at least one 32-column slab per compute unit take a second kernel that
 // needs none of that: K is split over the four waves of the workgroup (further down).
+#include <atomic>
+#include <cstdarg>
+#include <mutex>
+
 #include "epilogues.h"
 #include "mfma_tile.h"
 
@@ -587,4 +591,149 @@ bool launch_skinny_i8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const
   return true;
 }
 
+// ---- the entry point that allocates nothing --------------------------------------------------
+// For callers that cannot allocate device memory (code under HIP graph capture, tight serving
+// loops, harnesses that forbid it): the bf16 decode GEMM above with its split-K partials and
+// arrival counters in a file-scope device array instead of a handle's workspace, and no handle
+// (creating one allocates).  Each GPU the library runs on holds the array until the process
+// ends.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU race.
+namespace {
+
+constexpr size_t kStaticPartialBytes = (size_t)16 << 20;  // covers every N <= kStaticMaxN
+constexpr size_t kStaticCounterBytes = 4096;
+constexpr int64_t kStaticMaxN = 16384;
+constexpr int kStaticMaxDevices = 64;
+
+static __device__ __align__(256) unsigned char scratch[kStaticPartialBytes + kStaticCounterBytes];
+
+// `scratch` in host code is only a handle for the runtime's symbol table, not a device
+// address: the address of each device's copy is looked up once, with that device current.
+struct StaticDevice {
+  std::atomic<int> state{0};  // 0 = not looked up, 1 = ready, -1 = unusable (see status)
+  cigemmStatus_t status = CIGEMM_STATUS_SUCCESS;
+  char* ptr = nullptr;
+  int num_cus = 0;
+};
+StaticDevice g_static_dev[kStaticMaxDevices];
+std::mutex g_static_mutex;
+
+cigemmStatus_t static_device_setup(int dev, StaticDevice** out) {
+  StaticDevice& d = g_static_dev[dev];
+  if (d.state.load(std::memory_order_acquire) == 0) {
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (d.state.load(std::memory_order_relaxed) == 0) {
+      hipDeviceProp_t prop;
+      void* p = nullptr;
+      if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        d.status = CIGEMM_STATUS_NOT_INITIALIZED;
+      } else if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        d.status = CIGEMM_STATUS_ARCH_MISMATCH;
+      } else if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+        (void)hipGetLastError();
+        d.status = CIGEMM_STATUS_INTERNAL_ERROR;
+      } else {
+        d.ptr = static_cast<char*>(p);
+        d.num_cus = prop.multiProcessorCount;
+      }
+      d.state.store(d.status == CIGEMM_STATUS_SUCCESS ? 1 : -1, std::memory_order_release);
+    }
+  }
+  *out = &d;
+  return d.status;
+}
+
+// The arrival counters must be zero when the GEMM kernel starts.  A kernel, not a memset: this
+// call may be recorded into a graph.
+__global__ void clear_counters_kernel(uint32_t* counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0u;
+}
+
+cigemmStatus_t static_fail(char* err, size_t err_len, cigemmStatus_t st, const char* fmt, ...)
+    __attribute__((format(printf, 4, 5)));
+cigemmStatus_t static_fail(char* err, size_t err_len, cigemmStatus_t st, const char* fmt, ...) {
+  if (err && err_len) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(err, err_len, fmt, ap);
+    va_end(ap);
+  }
+  return st;
+}
+
+}  // namespace
 }  // namespace cig
+
+extern "C" cigemmStatus_t cigemm_gemm_bf16_static(void* stream, int64_t M, int64_t N, int64_t K,
+                                                  const uint16_t* A, int64_t lda,
+                                                  const uint16_t* B, int64_t ldb, uint16_t* C,
+                                                  int64_t ldc, char* err, size_t err_len) {
+  using namespace cig;
+  const char* name = "cigemm_gemm_bf16_static";
+  if (err && err_len) err[0] = '\0';
+  if (M < 0 || N < 0 || K < 0)
+    return static_fail(err, err_len, CIGEMM_STATUS_INVALID_VALUE,
+                       "%s: negative dimension (M=%lld N=%lld K=%lld)", name, (long long)M,
+                       (long long)N, (long long)K);
+  if (M == 0 || N == 0) return CIGEMM_STATUS_SUCCESS;
+  if (!A || !B || !C)
+    return static_fail(err, err_len, CIGEMM_STATUS_INVALID_VALUE, "%s: null pointer", name);
+  if (lda < K || ldb < N || ldc < N)
+    return static_fail(err, err_len, CIGEMM_STATUS_INVALID_VALUE,
+                       "%s: leading dimension too small (lda=%lld ldb=%lld ldc=%lld)", name,
+                       (long long)lda, (long long)ldb, (long long)ldc);
+  if (M > XROWS || N > kStaticMaxN)
+    return static_fail(err, err_len, CIGEMM_STATUS_NOT_SUPPORTED,
+                       "%s: M=%lld N=%lld beyond the maximum of this entry point (M <= %d, "
+                       "N <= %lld: its scratch memory is a fixed %zu-byte device array)",
+                       name, (long long)M, (long long)N, XROWS, (long long)kStaticMaxN,
+                       kStaticPartialBytes + kStaticCounterBytes);
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return static_fail(err, err_len, CIGEMM_STATUS_NOT_INITIALIZED, "%s: no HIP device", name);
+  }
+  if (dev < 0 || dev >= kStaticMaxDevices)
+    return static_fail(err, err_len, CIGEMM_STATUS_NOT_SUPPORTED, "%s: device %d >= %d", name,
+                       dev, kStaticMaxDevices);
+  StaticDevice* sd = nullptr;
+  const cigemmStatus_t st = static_device_setup(dev, &sd);
+  if (st != CIGEMM_STATUS_SUCCESS)
+    return static_fail(err, err_len, st, "%s: device %d cannot be used (%s)", name, dev,
+                       cigemmGetStatusString(st));
+
+  // a context on the stack, with the device array in the place of a handle's workspace
+  cigemmContext ctx{};
+  ctx.magic = kCtxMagic;
+  ctx.device = dev;
+  ctx.num_cus = sd->num_cus;
+  ctx.stream = static_cast<hipStream_t>(stream);
+  ctx.last_kernel = "";
+  ctx.algo = CIGEMM_ALGO_SKINNY;
+  ctx.workspace = sd->ptr;
+  ctx.ws_partial_bytes = kStaticPartialBytes;
+  ctx.ws_counter_bytes = kStaticCounterBytes;
+  typedef GeoKN16<tile::MathBF16> GB;
+  if (!skinny_shape_ok<GB>(&ctx, M, N, K, 2, A, lda, B, ldb) || ldc % 4 || ((uintptr_t)C & 7))
+    return static_fail(err, err_len, CIGEMM_STATUS_NOT_SUPPORTED,
+                       "%s: needs N %% 256 == 0, K %% 32 == 0, lda and ldb multiples of 8, ldc of "
+                       "4, A and B 16-byte and C 8-byte aligned (M=%lld N=%lld K=%lld)",
+                       name, (long long)M, (long long)N, (long long)K);
+  if (choose_splits<GB>(&ctx, N, K / GB::K_ELEMS) > 1) {
+    const int slabs = (int)(N / GB::BN);
+    hipLaunchKernelGGL(clear_counters_kernel, dim3((slabs + 255) / 256), dim3(256), 0, ctx.stream,
+                       reinterpret_cast<uint32_t*>(sd->ptr + kStaticPartialBytes), slabs);
+  }
+  launch_skinny<GB>(&ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<BF16>{C, ldc});
+  if (ctx.pending_error[0]) {
+    (void)hipGetLastError();
+    return static_fail(err, err_len, CIGEMM_STATUS_INTERNAL_ERROR, "%s: %s", name,
+                       ctx.pending_error);
+  }
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return static_fail(err, err_len, CIGEMM_STATUS_EXECUTION_FAILED, "%s: HIP error: %s", name,
+                       hipGetErrorString(e));
+  return CIGEMM_STATUS_SUCCESS;
+}

@@ -166,6 +166,27 @@ CIGEMM_API cigemmStatus_t cigemm_gemm_i8_dequant(
     cigemmScaleMode_t scaleA_mode, const float* scaleB, cigemmScaleMode_t scaleB_mode,
     void* out, cigemmOutType_t out_type, int64_t ldo, int32_t* acc_out, int64_t ldacc);
 
+/* bf16 GEMM for decode shapes that allocates nothing, anywhere: no handle, no workspace.
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid it; creating a
+ * handle allocates its workspace).  Same kernel and same results, bit for bit, as
+ * cigemm_gemm_bf16 on the same arguments; the kernel's scratch memory (split-K partial sums
+ * and arrival counters) is a fixed device array of 16 MiB + 4 KiB inside the library, which
+ * every GPU the process uses holds until the process ends.
+ *   Limits: 1 <= M <= 32, N <= 16384, N % 256 == 0, K % 32 == 0, lda and ldb multiples of 8,
+ *   ldc a multiple of 4, A and B 16-byte aligned, C 8-byte aligned; anything else returns
+ *   CIGEMM_STATUS_NOT_SUPPORTED (CIGEMM_STATUS_INVALID_VALUE for null pointers, negative sizes
+ *   or leading dimensions below the row length) and launches nothing.
+ *   `stream` is a hipStream_t passed as void* (NULL = the null stream); the call enqueues on
+ *   it, on the current device, and returns.  All calls on one GPU share that GPU's array:
+ *   calls that can overlap on one GPU (two streams, two threads) race on it.  The first call
+ *   on a device looks the array's address up and should happen outside graph capture.
+ *   `err` (may be NULL) receives the message of a failing call, at most err_len bytes. */
+CIGEMM_API cigemmStatus_t cigemm_gemm_bf16_static(void* stream, int64_t M, int64_t N, int64_t K,
+                                                  const uint16_t* A, int64_t lda,
+                                                  const uint16_t* B, int64_t ldb, uint16_t* C,
+                                                  int64_t ldc, char* err, size_t err_len);
+
 /* ---- linear layer: GEMM with bias and activation fused ------------------------------ */
 
 typedef enum cigemmActivation {

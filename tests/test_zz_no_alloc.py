@@ -1,0 +1,61 @@
+"""cigemm_gemm_bf16_static: the decode-shape bf16 GEMM that allocates nothing (no handle, its
+split-K scratch in a fixed device array inside the library), through the C ABI, against
+cigemm_gemm_bf16 on the same arguments.  Same kernel, same K ranges: the outputs must be
+identical bit for bit.  Two calls in a row share the device array, the second smaller."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import cudaintro_amd as ci
+from cudaintro_amd import workloads as wl
+from gpu_util import bits, error_bound_16, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def test_static_entry_matches_handle_entry_two_calls(handle, torch_gpu, oracle):
+    torch = torch_gpu
+    # first call: 32 column slabs x 8 K ranges fill 8 MiB of the array; second call: smaller
+    # in every dimension, 4 slabs x 16 ranges, over what the first call left behind
+    for (M, N, K) in [(8, 8192, 8192), (3, 1024, 2048)]:
+        xb, wb = wl.normal_16bit(M, N, K, seed=4 + M, kind="bf16", sigma_b=0.02)
+        x, w = to_dev(torch, xb, "bf16"), to_dev(torch, wb, "bf16")
+        y = torch.full((M + 2, N), 7.0, dtype=torch.bfloat16, device="cuda")
+        ci.gemm_bf16_static(x, w, out=y[:M])
+        with handle.algo(ci.ALGO_SKINNY):
+            y_ref = handle.gemm_bf16(x, w)
+        assert "skinny" in handle.last_kernel
+        got = bits(torch, y)
+        np.testing.assert_array_equal(got[:M], bits(torch, y_ref))
+        assert (got[M:] == oracle.f32_to_bf16(np.float32(7.0))).all()
+        # and against the fp64 checker on the rounded inputs
+        ref, S = oracle.gemm_f64(oracle.bf16_to_f32(xb), oracle.bf16_to_f32(wb), with_abs=True)
+        err = np.abs(oracle.bf16_to_f32(got[:M]).astype(np.float64) - ref)
+        assert (err <= error_bound_16(ref, S, K, "bf16")).all()
+
+
+def test_static_entry_rejects_what_it_cannot_hold(torch_gpu):
+    torch = torch_gpu
+    x = torch.zeros((33, 64), dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros((64, 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ci.CigemmError) as e:
+        ci.gemm_bf16_static(x, w)
+    assert e.value.status == ci.Status.NOT_SUPPORTED and "maximum" in str(e.value)
+    x = torch.zeros((1, 64), dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros((64, 16384 + 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ci.CigemmError) as e:
+        ci.gemm_bf16_static(x, w)
+    assert e.value.status == ci.Status.NOT_SUPPORTED and "16384" in str(e.value)
+    # a shape outside the kernel's gate, and bad arguments: a code, no launch
+    w = torch.zeros((64, 128), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ci.CigemmError) as e:
+        ci.gemm_bf16_static(x, w)
+    assert e.value.status == ci.Status.NOT_SUPPORTED
+    lib = ci.load_library()
+    err = ctypes.create_string_buffer(128)
+    st = lib.cigemm_gemm_bf16_static(None, 1, 256, 64, None, 64, None, 256, None, 256, err, 128)
+    assert st == ci.Status.INVALID_VALUE and b"null" in err.value
+    st = lib.cigemm_gemm_bf16_static(None, 0, 256, 64, None, 64, None, 256, None, 256, None, 0)
+    assert st == ci.Status.SUCCESS
+    torch.cuda.synchronize()
