@@ -188,6 +188,57 @@ def cpu_rows_baseline(run_rows, M, ops_per_row, unit, what, target_seconds=3.0):
             "kind": "port", "sample": f"first {rows2} of {M} rows of the same problem, {what}, {dt:.2f} s"}, res
 
 
+def k_sweep(torch, ci, wl, handle, steps, warmup):
+    """Per-launch time of the tile kernel at several K for a fixed M x N, and the least-squares
+    fit t = rounds * (a + b * stages): `a` is what one output tile costs whatever its K
+    (pipeline fill, epilogue, the burst of output stores), `b` the cost of one 64-byte stage
+    of k.  Prints one JSON object."""
+    res = {}
+
+    def fit(rows, cus=256):
+        # rows: (K stages, tiles, seconds per launch)
+        x = np.array([[np.ceil(t / cus), np.ceil(t / cus) * st] for st, t, _ in rows], np.float64)
+        y = np.array([sec for _, _, sec in rows], np.float64)
+        (a, b), *_ = np.linalg.lstsq(x, y, rcond=None)
+        return a * 1e6, b * 1e6
+
+    for name, sz, ks in (("int8_kn_dequant_f32_4096x4096", 4096, (1024, 2048, 4096, 8192)),
+                         ("int8_kn_raw_i32_8192x8192", 8192, (2048, 4096, 8192)),
+                         ("bf16_4096x4096", 4096, (1024, 2048, 4096, 8192)),
+                         ("bf16_8192x8192", 8192, (2048, 4096, 8192))):
+        kmax = max(ks)
+        rows = []
+        if name.startswith("int8"):
+            Aq, Bq, sa, sb = wl.int8_uniform(sz, sz, kmax, seed=1)
+            a, b = torch.from_numpy(Aq).cuda(), torch.from_numpy(Bq).cuda()
+            sa_d, sb_d = torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda()
+            deq = "dequant" in name
+            out = torch.empty((sz, sz), device="cuda", dtype=torch.float32 if deq else torch.int32)
+            for K in ks:
+                av, bv = a[:, :K], b[:K]
+                if deq:
+                    fn = lambda: handle.gemm_i8_dequant(av, bv, sa_d, sb_d, ci.B_KN, ci.OUT_F32, out=out)  # noqa: E731
+                else:
+                    fn = lambda: handle.gemm_i8_i32(av, bv, ci.B_KN, out=out)  # noqa: E731
+                _, e = time_calls(torch, fn, steps, warmup)
+                rows.append((K // 64, (sz // 256) ** 2, e / steps))
+                res.setdefault(name, {})[f"K{K}"] = {"us": e / steps * 1e6, "kernel": handle.last_kernel}
+        else:
+            Ab, Bb = wl.normal_16bit(sz, sz, kmax, seed=2, kind="bf16")
+            a, b = dev16(torch, Ab, "bf16"), dev16(torch, Bb, "bf16")
+            out = torch.empty((sz, sz), dtype=torch.bfloat16, device="cuda")
+            for K in ks:
+                av, bv = a[:, :K], b[:K]
+                _, e = time_calls(torch, lambda: handle.gemm_bf16(av, bv, out=out), steps, warmup)
+                rows.append((K // 32, (sz // 256) ** 2, e / steps))
+                res.setdefault(name, {})[f"K{K}"] = {"us": e / steps * 1e6, "kernel": handle.last_kernel}
+        a_us, b_us = fit(rows)
+        res[name]["fit"] = {"a_us_per_tile": a_us, "b_us_per_stage": b_us}
+        log(f"[k-sweep] {name}: {json.dumps(res[name])}")
+        del a, b, out
+    print(json.dumps({"k_sweep": res}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -205,6 +256,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy a few times (reference point for "
                          "the FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
+    ap.add_argument("--k-sweep", action="store_true",
+                    help="instead of the benchmark: time the tile kernel at several K per M x N and "
+                         "fit its fixed cost per tile and its cost per stage")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1",
@@ -219,6 +273,9 @@ def main():
         print("bench.py needs an MI355X; there is no CPU fallback", file=sys.stderr)
         sys.exit(1)
     handle = ci.Handle()
+    if args.k_sweep:
+        k_sweep(torch, ci, wl, handle, args.steps, args.warmup)
+        return
     n = args.size
     per_config = {}
     mfma_probe = {}

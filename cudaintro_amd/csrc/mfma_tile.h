@@ -123,9 +123,14 @@ struct RowMajorDmaT {
 };
 typedef RowMajorDmaT<4> RowMajorDma;
 
+// Source of the 16-byte pieces that lie past the end of K in the last stage: the matrix
+// instructions always consume whole 64-byte stages, so what K does not fill is fetched from here.
+static __device__ __align__(64) uint32_t g_zero_chunk[16];
+
 // Weights N x K: identical to the A tile.
 template <>
 struct BTile<B_NK> : RowMajorDma, HalfPieces {
+  static __device__ __forceinline__ int dma_k(int, int, int) { return 0; }  // (fetched as pairs)
   // half h (0/1) of the fragment of column tile j, k-step kk: 8 bytes of k
   static __device__ __forceinline__ u32x2 frag_half(const char* sb, int wn, int j, int kk, int h,
                                                     int l) {
@@ -150,6 +155,8 @@ struct BTile<B_KN16> : HalfPieces {
   }
   static __device__ __forceinline__ int off(int k, int c) { return k * 512 + ((c ^ swz(k)) << 4); }
   static __device__ __forceinline__ int dma_lds(int w, int i) { return (8 * w + 2 * i) * 512; }
+  // k row (within the stage) that lane l of instruction (w, i) fetches
+  static __device__ __forceinline__ int dma_k(int w, int i, int l) { return 8 * w + 2 * i + (l >> 5); }
   // `last` = last valid 16-byte chunk of a tile row (columns beyond N re-read it)
   static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld, int last) {
     const int k = 8 * w + 2 * i + (l >> 5);
@@ -174,6 +181,7 @@ struct BTile<B_KN8> : HalfPieces {
   }
   static __device__ __forceinline__ int off(int k, int c) { return k * 256 + ((c ^ swz(k)) << 4); }
   static __device__ __forceinline__ int dma_lds(int w, int i) { return (16 * w + 4 * i) * 256; }
+  static __device__ __forceinline__ int dma_k(int w, int i, int l) { return 16 * w + 4 * i + (l >> 4); }
   static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld, int last) {
     const int k = 16 * w + 4 * i + (l >> 4);
     const int c = (l & 15) ^ swz(k);
@@ -198,6 +206,7 @@ struct BTile<B_KN32> {
   typedef uint32_t piece_t;
   static __device__ __forceinline__ int swz(int k) { return ((k >> 2) & 1) << 3; }
   static __device__ __forceinline__ int dma_lds(int w, int i) { return (4 * w + i) * 1024; }
+  static __device__ __forceinline__ int dma_k(int w, int i, int) { return 4 * w + i; }
   static __device__ __forceinline__ int64_t dma_src(int w, int i, int l, int64_t ld, int last) {
     const int k = 4 * w + i;
     const int c = l ^ swz(k);
@@ -352,10 +361,11 @@ __device__ __forceinline__ EpiPartialX4 epilogue_of_split(const EpiPartialX4& e,
 //
 // A, B are byte pointers; lda/ldb are in BYTES.  Any M; N a multiple of 4; all rows 16-byte
 // aligned (tile_shape_ok checks).  KTS = number of 64-byte stages of this workgroup's K
-// range; grid = (tiles, K ranges).
+// range, k_bytes = bytes of k in it (a multiple of 16; the last stage may be partly filled:
+// the pieces past k_bytes are fetched as zeros); grid = (tiles, K ranges).
 template <typename Math, int BMODE, int NSTAGES, int MT, typename Epi, int WM = 2>
 __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, int tiles_m,
-                                                           int tiles_n, int KTS,
+                                                           int tiles_n, int KTS, int k_bytes,
                                                            const char* __restrict__ A,
                                                            int64_t lda,
                                                            const char* __restrict__ B,
@@ -422,26 +432,15 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   const int a_last = (int)((M - 1 - m0) < (TILE_M - 1) ? (M - 1 - m0) : (TILE_M - 1));
   const int n_left = (int)((N - n0) < BN ? (N - n0) : BN);
   const int b_last = BMODE == B_NK ? n_left - 1 : n_left * Math::ELEM_BYTES / 16 - 1;
-  // With an odd number of stages the last pair's second half lies past this K range (past
-  // the end of A for the last rows of the matrix): lanes that would fetch it fetch the first
-  // half again instead (bit i of a_hi = instruction i of this lane fetches chunk 4..7); that
-  // half of the slot is never read.
-  uint32_t a_hi = 0;
-#pragma unroll
-  for (int i = 0; i < DMA_A; ++i) {
-    const int r = 8 * (DMA_A * w + i) + (l >> 3);
-    a_hi |= (uint32_t)((((l & 7) ^ pair_swz(r)) >> 2) & 1) << i;
-  }
+  // The last pair of stages may be filled only in part (an odd number of stages, or a K that
+  // does not fill its last stage): pair_valid = 16-byte pieces of it that lie inside this K
+  // range (1..8), tail_k = bytes of k inside the last stage (16..64).  What lies beyond is
+  // fetched from a block of zeros instead (reading on would leave the row, and for the last
+  // rows the matrix), so the matrix instructions see zero operands there.
   const int last_pair = (KTS - 1) >> 1;
-  const bool odd_kts = KTS & 1;
-  uint32_t b_hi = 0;  // the same for the rows of N x K weights
-  if (BPAIR) {
-#pragma unroll
-    for (int i = 0; i < DMA_B; ++i) {
-      const int r = 8 * (DMA_B * w + i) + (l >> 3);
-      b_hi |= (uint32_t)((((l & 7) ^ pair_swz(r)) >> 2) & 1) << i;
-    }
-  }
+  const int pair_valid = (k_bytes - last_pair * 128) >> 4;
+  const int tail_k = k_bytes - (KTS - 1) * KB;
+  const char* const zero_src = reinterpret_cast<const char*>(g_zero_chunk);
   uint32_t a_voff[DMA_A], b_voff[DMA_B];
 #pragma unroll
   for (int i = 0; i < DMA_A; ++i) {
@@ -471,6 +470,16 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
                  : "s"(lds_dst), "v"(voff), "s"(base)
                  : "m0");
   };
+  // the same with a full per-lane address: lanes with `zero` set fetch zeros
+  auto dma16z = [&](const char* base, uint32_t voff, uint32_t lds_dst, bool zero) {
+    const char* src = zero ? zero_src : base + voff;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_dst), "v"(src)
+                 : "m0");
+  };
+  // piece (16 bytes of k) that lane l fetches with pair instruction q (rows 8 q .. 8 q + 7)
+  auto pair_piece = [&](int q) { return (l & 7) ^ ((4 * (q & 1) + (l >> 4)) & 7); };
   // d < DMA_B: B instruction d of stage `st` (of its stage pair, for N x K weights) into B
   // slot `slot`; above: A instruction d - DMA_B of the stage pair st / 2 into pair slot `pslot`.
   // Past the last stage the last one is fetched
@@ -481,25 +490,30 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   auto dma_piece = [&](int st, int slot, int pslot, int d, auto steady_const) {
     constexpr bool STEADY = decltype(steady_const)::value;
     if (!STEADY) st = st < KTS ? st : KTS - 1;
-    const bool tail_pair = !STEADY && odd_kts && (st >> 1) == last_pair;
+    const bool part_pair = !STEADY && pair_valid < 8 && (st >> 1) == last_pair;
     if (d < DMA_B) {
+      const int q = DMA_B * w + d;
       if (BPAIR) {
-        uint32_t off = b_voff[d];
-        if (tail_pair) off -= ((b_hi >> d) & 1u) << 6;
-        const int q = DMA_B * w + d;
-        dma16(b_tile + (int64_t)(st >> 1) * 128, off,
-              lds_base + slot * BPAIR_BYTES + PairDma::dma_lds(q >> 1, q & 1));
+        const uint32_t dst = lds_base + slot * BPAIR_BYTES + PairDma::dma_lds(q >> 1, q & 1);
+        if (part_pair)
+          dma16z(b_tile + (int64_t)(st >> 1) * 128, b_voff[d], dst, pair_piece(q) >= pair_valid);
+        else
+          dma16(b_tile + (int64_t)(st >> 1) * 128, b_voff[d], dst);
       } else {
-        const int q = DMA_B * w + d;
-        dma16(b_tile + (int64_t)st * b_kstep, b_voff[d],
-              lds_base + slot * OPERAND_BYTES + BT::dma_lds(q >> 2, q & 3));
+        const uint32_t dst = lds_base + slot * OPERAND_BYTES + BT::dma_lds(q >> 2, q & 3);
+        if (!STEADY && tail_k < KB && st == KTS - 1)
+          dma16z(b_tile + (int64_t)st * b_kstep, b_voff[d], dst,
+                 BT::dma_k(q >> 2, q & 3, l) * Math::ELEM_BYTES >= tail_k);
+        else
+          dma16(b_tile + (int64_t)st * b_kstep, b_voff[d], dst);
       }
     } else {
-      uint32_t off = a_voff[d - DMA_B];
-      if (tail_pair) off -= ((a_hi >> (d - DMA_B)) & 1u) << 6;
-      dma16(a_tile + (int64_t)(st >> 1) * 128, off,
-            lds_base + B_RING + pslot * APAIR_BYTES +
-                PairDma::dma_lds((DMA_A * w + d - DMA_B) >> 1, (DMA_A * w + d - DMA_B) & 1));
+      const int q = DMA_A * w + d - DMA_B;
+      const uint32_t dst = lds_base + B_RING + pslot * APAIR_BYTES + PairDma::dma_lds(q >> 1, q & 1);
+      if (part_pair)
+        dma16z(a_tile + (int64_t)(st >> 1) * 128, a_voff[d - DMA_B], dst, pair_piece(q) >= pair_valid);
+      else
+        dma16(a_tile + (int64_t)(st >> 1) * 128, a_voff[d - DMA_B], dst);
     }
   };
   typedef std::integral_constant<bool, true> steady_t;
@@ -664,9 +678,10 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
       dma_pslot = dma_pslot + 1 == 3 ? 0 : dma_pslot + 1;
     }
   };
-  // Steady part: every stage the DMA reaches (up to s + 5) exists and is not the odd tail.
+  // Steady part: every stage the DMA reaches (up to s + 5) exists and its pair is whole.
+  const int steady_end = (pair_valid < 8 && !(KTS & 1)) ? KTS - 2 : KTS;
   int s = 0;
-  for (; s + 5 < KTS; s += 2) {
+  for (; s + 5 < steady_end; s += 2) {
     stage(s, std::integral_constant<int, 0>{}, steady_t{});
     stage(s + 1, std::integral_constant<int, 1>{}, steady_t{});
   }

@@ -39,3 +39,23 @@ def handle(torch_gpu):
 @pytest.fixture
 def rng():
     return np.random.Generator(np.random.PCG64(12345))
+
+
+@pytest.fixture(scope="session")
+def parity_stats():
+    """Observed error figures of the configuration tests (errors in units of the bound each
+    test gates on, bit-exactness verdicts).  Written as JSON next to the other outputs of a GPU
+    run when the session ends, so that a run leaves the measured numbers behind and not only
+    pass/fail."""
+    import json
+    stats = {}
+    yield stats
+    if not stats:
+        return
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out_dir, exist_ok=True)
+        with open(os.path.join(out_dir, "parity_stats.json"), "w") as f:
+            json.dump(stats, f, indent=1, sort_keys=True)
+    except OSError:
+        pass

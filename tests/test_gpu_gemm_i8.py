@@ -80,7 +80,7 @@ def test_dequant_bit_exact(handle, torch_gpu, oracle, rng, b_nk, out_type, modes
     assert torch_gpu.equal(out, out2)
 
 
-def test_config_int8_4096(handle, torch_gpu, oracle):
+def test_config_int8_4096(handle, torch_gpu, oracle, parity_stats):
     """int8 4096^3, uniform [-127,127] seed 1, per-tensor scales 1/127, fp32 out."""
     A, B, sa, sb = wl.int8_uniform(4096, 4096, 4096, seed=1)
     out, acc = handle.gemm_i8_dequant(dev(torch_gpu, A), dev(torch_gpu, B), dev(torch_gpu, sa),
@@ -91,9 +91,11 @@ def test_config_int8_4096(handle, torch_gpu, oracle):
     np.testing.assert_array_equal(out.cpu().numpy(), oracle.dequant(acc_ref, sa, sb))
     raw = handle.gemm_i8_i32(dev(torch_gpu, A), dev(torch_gpu, B))
     np.testing.assert_array_equal(raw.cpu().numpy(), acc_ref)
+    parity_stats["C2_int8_4096_dequant_f32"] = {"accumulators_bit_exact": True, "outputs_bit_exact": True,
+                                               "entries_compared": int(acc_ref.size)}
 
 
-def test_config_quantized_linear(handle, torch_gpu, oracle):
+def test_config_quantized_linear(handle, torch_gpu, oracle, parity_stats):
     """Prefill-shaped quantized linear: M=2048, K=4096, N=11008, per-row x per-channel
     scales, bf16 out."""
     Xq, sx, Wq, sw = wl.quantized_linear(2048, 4096, 11008, seed=3)
@@ -103,6 +105,9 @@ def test_config_quantized_linear(handle, torch_gpu, oracle):
     acc_ref = oracle.gemm_i8_i32(Xq, Wq, b_is_nk=True)
     np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
     np.testing.assert_array_equal(bits(torch_gpu, out), oracle.dequant(acc_ref, sx, sw, out_dtype="bf16"))
+    parity_stats["C4_int8_linear_2048x11008x4096_bf16"] = {
+        "kernel": handle.last_kernel, "accumulators_bit_exact": True, "outputs_bit_exact": True,
+        "entries_compared": int(acc_ref.size)}
 
 
 def test_quantize_then_gemm_device_pipeline(handle, torch_gpu, oracle, rng):

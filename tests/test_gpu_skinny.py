@@ -130,7 +130,7 @@ def test_skinny_int8_without_split_k(handle, torch_gpu, oracle, rng, M, N, K):
         np.testing.assert_array_equal(got, expect)
 
 
-def test_config_skinny_decode(handle, torch_gpu, oracle):
+def test_config_skinny_decode(handle, torch_gpu, oracle, parity_stats):
     """The decode-shaped configurations: M in {1, 8, 32}, N = K = 8192, bf16 weights N(0,0.02)
     and int8 weights with per-channel scales."""
     torch = torch_gpu
@@ -140,7 +140,11 @@ def test_config_skinny_decode(handle, torch_gpu, oracle):
         assert "skinny" in handle.last_kernel
         ref, S = oracle.gemm_f64(oracle.bf16_to_f32(xb), oracle.bf16_to_f32(wb), with_abs=True)
         got = oracle.bf16_to_f32(bits(torch, y)).astype(np.float64)
-        assert (np.abs(got - ref) <= error_bound_16(ref, S, 8192, "bf16")).all()
+        ratio = np.abs(got - ref) / error_bound_16(ref, S, 8192, "bf16")
+        parity_stats[f"C5_skinny_bf16_M{M}"] = {"kernel": handle.last_kernel,
+                                                "max_err_over_bound": float(ratio.max()),
+                                                "mean_err_over_bound": float(ratio.mean())}
+        assert (ratio <= 1.0).all()
         xq, sx, wq, sw = wl.skinny_int8(M, 8192, 8192, seed=4)
         out, acc = handle.gemm_i8_dequant(torch.from_numpy(xq).cuda(), torch.from_numpy(wq).cuda(),
                                           torch.from_numpy(sx).cuda(), torch.from_numpy(sw).cuda(),
@@ -150,6 +154,8 @@ def test_config_skinny_decode(handle, torch_gpu, oracle):
         np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
         np.testing.assert_array_equal(bits(torch, out),
                                       oracle.dequant(acc_ref, sx, sw, out_dtype="bf16", sa_per_row=M > 1))
+        parity_stats[f"C5_skinny_int8_M{M}"] = {"kernel": handle.last_kernel,
+                                                "accumulators_bit_exact": True, "outputs_bit_exact": True}
 
 
 @pytest.mark.parametrize("shape", [(5, 1024, 2048), (8, 8192, 8192)])
