@@ -10,7 +10,7 @@ namespace cig {
 bool launch_16b_mfma(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_t K,
                      const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, uint16_t* C,
                      int64_t ldc) {
-  if (!tile::tile_shape_ok(M, N, K, 2, A, lda, B, ldb, true) || N % 8) return false;
+  if (!tile::tile_shape_ok(M, N, K, 2, A, lda, B, ldb, true)) return false;
   if (ldc % 8 || ((uintptr_t)C & 15)) return false;  // output rows are stored in 16-byte pieces
   if (bf16) {
     const bool split = tile::launch_tile<tile::MathBF16, tile::B_KN16>(

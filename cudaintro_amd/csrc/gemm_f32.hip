@@ -32,7 +32,7 @@ bool launch_f32_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const 
     const bool one_round = ((M + 255) / 256) * ((N + tile::BN - 1) / tile::BN) <= cus;
     const bool long_k_split =
         tile_ok && K >= 2048 && one_round &&
-        tile::plan_small(ctx, M, N, K * 4 / tile::KB, tile::MathF32::STAGE_UNIT_US, K * 4 * N)
+        tile::plan_small(ctx, M, N, K * 4, tile::MathF32::STAGE_UNIT_US, K * 4 * N)
                 .splits > 1;
     if (!tile_ok || (small_cost < tile_cost && !long_k_split)) {
       launch_f32_small(ctx, M, N, K, A, lda, B, ldb, C, ldc, ba);

@@ -35,7 +35,6 @@ bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const i
                     int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C, int64_t ldc,
                     const DequantArgs* dq) {
   if (!tile::tile_shape_ok(M, N, K, 1, A, lda, B, ldb, !b_nk)) return false;
-  if (dq && dq->out_bf16 && N % 8) return false;
   if (!dq) {
     if (ldc % 4 || ((uintptr_t)C & 15)) return false;
   } else {

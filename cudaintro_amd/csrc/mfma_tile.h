@@ -431,7 +431,7 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   // is never stored.
   const int a_last = (int)((M - 1 - m0) < (TILE_M - 1) ? (M - 1 - m0) : (TILE_M - 1));
   const int n_left = (int)((N - n0) < BN ? (N - n0) : BN);
-  const int b_last = BMODE == B_NK ? n_left - 1 : n_left * Math::ELEM_BYTES / 16 - 1;
+  const int b_last = BMODE == B_NK ? n_left - 1 : (n_left * Math::ELEM_BYTES + 15) / 16 - 1;
   // The last pair of stages may be filled only in part (an odd number of stages, or a K that
   // does not fill its last stage): pair_valid = 16-byte pieces of it that lie inside this K
   // range (1..8), tail_k = bytes of k inside the last stage (16..64).  What lies beyond is
@@ -699,9 +699,10 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   // holds short pieces of 32 different rows.  Each wave stages one 32-row x 128-column block
   // at a time in its own piece of the (now idle) LDS and writes it out as whole rows: every
   // store instruction then covers full 256- or 512-byte row segments.
-  // The lane number as the epilogue sees it is opaque to the compiler, so that none of the
-  // epilogue's addresses is computed ahead and held in a register through the main loop.
-  int le = l;
+  // The epilogue takes the lane number afresh from the hardware (and opaque to the compiler),
+  // so that neither it nor any of the epilogue's addresses is held in a register through the
+  // main loop.
+  int le = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
   asm volatile("" : "+v"(le));
   le &= 63;
   const int ge = le >> 5;
@@ -767,11 +768,17 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
       const int rl = p * ROWS_PER_PASS + le / LANES_PER_ROW;
       const int c16 = le % LANES_PER_ROW;
       const u32x4 v = *reinterpret_cast<const u32x4*>(scr + rl * ROW_STRIDE + c16 * 16);
-      // N * OB is a multiple of 16: a 16-byte piece is in or out as a whole
-      if (row0 + rl < M && n0 + wn * 128 + c16 * (16 / OB) < N)
-        // streaming store: C is not read again by this kernel and should not evict A / B
-        __builtin_nontemporal_store(
-            v, reinterpret_cast<u32x4*>(epi.out_row(row0 + rl) + (n0 + wn * 128) * OB + c16 * 16));
+      // N is a multiple of 4: a 16-byte piece of 32-bit outputs is in or out as a whole, one
+      // of 16-bit outputs may be half inside (then its first 8 bytes are stored)
+      const int64_t piece_col = n0 + wn * 128 + c16 * (16 / OB);
+      if (row0 + rl < M && piece_col < N) {
+        char* dst = epi.out_row(row0 + rl) + (n0 + wn * 128) * OB + c16 * 16;
+        // streaming stores: C is not read again by this kernel and should not evict A / B
+        if (OB == 2 && piece_col + 8 > N)
+          __builtin_nontemporal_store(u32x2{v[0], v[1]}, reinterpret_cast<u32x2*>(dst));
+        else
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
+      }
     }
   }
 }
@@ -794,11 +801,14 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
   ctx->last_tile_rows = TILE_M;
   ctx->last_k_splits = splits;
   ctx->last_waves = 2 * WM;
-  const int64_t kts = K_bytes / KB / splits;  // stages per K range
+  // stages per K range; only an unsplit K may leave its last stage partly filled
+  const int64_t kts = splits > 1 ? K_bytes / KB / splits : (K_bytes + KB - 1) / KB;
+  const int64_t range_bytes = splits > 1 ? kts * KB : K_bytes;
   const int64_t a_step = kts * KB;
   const int64_t b_step = BMODE == B_NK ? kts * KB : kts * (KB / Math::ELEM_BYTES) * ldb_bytes;
   hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(128 * WM),
                      LDS_BYTES, ctx->stream, (int)M, (int)N, tiles_m, tiles_n, (int)kts,
+                     (int)range_bytes,
                      static_cast<const char*>(A), lda_bytes, static_cast<const char*>(B),
                      ldb_bytes, epi, a_step, b_step);
 }
@@ -856,8 +866,10 @@ inline double tile_cost_units(int mt, bool streamed) {
   return streamed ? 1.2 + 0.7 * mt : 0.8 + 0.8 * mt;
 }
 
-inline SmallPlan plan_small(const cigemmContext* ctx, int64_t M, int64_t N, int64_t kts,
+inline SmallPlan plan_small(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes,
                             double sm_us, int64_t b_bytes) {
+  const int64_t kts = (K_bytes + KB - 1) / KB;
+  const bool whole_stages = K_bytes % KB == 0;  // K ranges are whole stages
   const bool streamed = b_bytes > (16LL << 20);
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
   SmallPlan best{0, 1};
@@ -868,7 +880,7 @@ inline SmallPlan plan_small(const cigemmContext* ctx, int64_t M, int64_t N, int6
     const double per_tile = tile_cost_units(mt, streamed);
     for (int sp = 1; sp <= 16; sp *= 2) {
       if (sp > 1) {
-        if (!ctx->workspace || kts % sp || kts / sp < 8) break;
+        if (!ctx->workspace || !whole_stages || kts % sp || kts / sp < 8) break;
         if ((size_t)sp * (size_t)M * (size_t)N * 4 > ctx->ws_partial_bytes) break;
       }
       const double rounds = (double)((tiles * sp + cus - 1) / cus);
@@ -985,7 +997,7 @@ bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
     // At most one round of 256-row tiles: pick the tile height and the number of K ranges
     // together.  Split plans run K over blockIdx.y, partial sums to the workspace, then one
     // reduction launch with the real epilogue.
-    const SmallPlan plan = plan_small(ctx, M, N, K_bytes / KB, Math::STAGE_UNIT_US, K_bytes * N);
+    const SmallPlan plan = plan_small(ctx, M, N, K_bytes, Math::STAGE_UNIT_US, K_bytes * N);
     if (plan.splits > 1) {
       typedef typename Math::scalar_t scalar_t;
       uint32_t* ws = static_cast<uint32_t*>(ctx->workspace);
@@ -1031,15 +1043,15 @@ bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
 }
 
 // Shape / alignment gate shared by the families (sizes in elements, elem = bytes each;
-// b_kn = B is K x N).  M is free; K must fill whole 64-byte stages (nothing pads k with
-// zeros); N must keep 16-byte pieces whole, on the input side (K x N rows) and on the output
-// side (the caller checks its output type).  Per-lane DMA offsets are 32-bit: 256 rows of
-// either operand must span less than 2 GiB.
+// b_kn = B is K x N).  M is free; K must fill whole 16-byte pieces (a last stage of fewer
+// than four is completed with zeros); N a multiple of 4 (a last 16-byte piece of a K x N row
+// that is only partly inside the matrix is still read whole: its row is 16-byte aligned, so the
+// piece cannot leave the page that holds its first byte).  Per-lane DMA offsets are 32-bit: 256
+// rows of either operand must span less than 2 GiB.
 inline bool tile_shape_ok(int64_t M, int64_t N, int64_t K, int elem, const void* A, int64_t lda,
                           const void* B, int64_t ldb, bool b_kn) {
   if (M <= 0 || N <= 0 || K <= 0) return false;
-  if ((K * elem) % KB || N % 4) return false;
-  if (b_kn && (N * elem) % 16) return false;
+  if ((K * elem) % 16 || N % 4) return false;
   if (M > 2147483647LL || N > 2147483647LL) return false;
   if ((lda * elem) % 16 || (ldb * elem) % 16) return false;
   if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return false;
