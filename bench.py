@@ -303,6 +303,15 @@ def main():
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_16BIT_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_16BIT_TFLOPS, "traffic": None, "kernel": kernel,
                 "avg_kernel_ms": ev / args.steps * 1e3}
+    # where the time of one launch goes, from timestamps inside the kernel (one instrumented
+    # launch of the same kernel, taken while the chip is in the state the timed loop left)
+    for _ in range(3):
+        phases = handle.probe_tile_phases(A, B, C)
+    roofline["phases"] = phases
+    roofline["clock_ghz_main_loop_this_run"] = phases["main_loop_clock_ghz"]
+    # matrix-core issue cycles of one 64-byte stage of the 256 x 256 tile: 32 instructions of 8
+    # passes of 4 cycles per wave
+    roofline["mfma_issue_fraction_of_main_loop"] = 1024.0 / phases["cycles_per_stage"]
     roofline["median_kernel_ms"] = median_call_ms(torch, lambda: handle.gemm_bf16(A, B, out=C),
                                                   max(50, args.steps))
     # HBM-side bytes per launch and the counter decomposition of the same kernel are not
@@ -350,6 +359,21 @@ def main():
 
         log(f"[bench] fp16 {n}^3")
         per_config[f"fp16_{n}"] = run16("f16")
+
+        # shapes that do not fill the kernel's units: a K whose last 64-byte stage holds one
+        # 16-byte piece, an N whose last column tile holds 8 columns (no alignment cliff wanted)
+        for (Mx, Nx, Kx) in ((n, n, n + 8), (n, n + 8, n)):
+            a_b, b_b = wl.normal_16bit(Mx, Nx, Kx, seed=2, kind="bf16")
+            a, b = dev16(torch, a_b, "bf16"), dev16(torch, b_b, "bf16")
+            c = torch.empty((Mx, Nx), dtype=torch.bfloat16, device="cuda")
+            steps_x = max(10, args.steps // 4)
+            w, e = time_calls(torch, lambda: handle.gemm_bf16(a, b, out=c), steps_x, max(5, args.warmup // 4))
+            t = wl.gemm_ops(Mx, Nx, Kx) * steps_x / e / 1e12
+            per_config[f"bf16_{Mx}x{Nx}x{Kx}"] = {"tflops": t, "frac_of_peak": t / PEAK_16BIT_TFLOPS,
+                                                   "peak": PEAK_16BIT_TFLOPS, "ms": e / steps_x * 1e3,
+                                                   "ms_over_aligned": e / steps_x / (ev / args.steps),
+                                                   "kernel": handle.last_kernel}
+            del a, b, c
         per_config[f"bf16_{n}"] = {"tflops": achieved, "frac_of_peak": achieved / PEAK_16BIT_TFLOPS,
                                    "peak": PEAK_16BIT_TFLOPS, "ms": ev / args.steps * 1e3,
                                    "kernel": kernel}
@@ -370,6 +394,14 @@ def main():
             t = wl.gemm_ops(M, N, K) * args.steps / e / 1e12
             per_config[name] = {"tops": t, "frac_of_peak": t / PEAK_INT8_TOPS, "peak": PEAK_INT8_TOPS,
                                 "ms": e / args.steps * 1e3, "kernel": handle.last_kernel}
+            if lay == ci.B_KN:
+                # phases of the same tile kernel with raw int32 output (the same bytes per
+                # output element as the fp32 dequantized one)
+                o32 = out if not dequant else torch.empty((M, N), dtype=torch.int32, device="cuda")
+                for _ in range(3):
+                    ph = handle.probe_tile_phases(a, b, o32)
+                per_config[name]["phases_raw_i32_out"] = ph
+                del o32
             if not args.no_cpu:
                 # the int8 -> int32 twin of the reference's CPU loop on a slice of rows, timed;
                 # the same rows of the GPU result are compared with it (bit-exact or not)

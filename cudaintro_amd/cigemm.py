@@ -75,6 +75,8 @@ SIGNATURES = {
     "cigemm_matrixMulMatrixCores": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
     "cigemm_matrixMulMatrixCoresBfloat16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
     "cigemm_probe_mfma": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int64)]),
+    "cigemm_probe_tile_phases": (C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp,
+                                           _i64, C.POINTER(C.c_double)]),
     "cigemmSetAlgo": (C.c_int, [_vp, C.c_int]),
     "cigemmGetAlgo": (C.c_int, [_vp, C.POINTER(C.c_int)]),
     "cigemm_gemm_f32": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
@@ -268,6 +270,21 @@ class Handle:
         self._check(self.lib.cigemm_probe_mfma(self._h, k, int(random_bits), iters, C.byref(ops)),
                     "cigemm_probe_mfma")
         return ops.value
+
+    def probe_tile_phases(self, A, B, out):
+        """One instrumented launch of the 256-row tile kernel (bf16 or int8 K x N -> int32);
+        returns the phase figures as a dict (see cigemm_probe_tile_phases)."""
+        torch = _torch()
+        kind = {torch.bfloat16: 0, torch.int8: 1}[A.dtype]
+        M, K = A.shape
+        N = B.shape[1]
+        ph = (C.c_double * 8)()
+        st = self.lib.cigemm_probe_tile_phases(self._h, kind, M, N, K, A.data_ptr(), self._ld(A),
+                                               B.data_ptr(), self._ld(B), out.data_ptr(), self._ld(out), ph)
+        self._check(st, "cigemm_probe_tile_phases")
+        keys = ("prologue_us", "main_loop_us", "epilogue_us", "first_start_to_last_end_us",
+                "cycles_per_stage", "main_loop_clock_ghz", "first_epilogue_to_last_end_us", "workgroups")
+        return dict(zip(keys, list(ph)))
 
     # -- study kernels (TileProgramming demo) -------------------------------------------------
     def matrixMulTiled(self, A, B):

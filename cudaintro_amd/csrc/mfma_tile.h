@@ -350,6 +350,20 @@ template <typename E>
 struct epi_has_uniform_mode<E, typename std::enable_if<E::HAS_UNIFORM_MODE>::type>
     : std::true_type {};
 
+// Measurement aid: an epilogue that declares `static constexpr bool PROFILED = true` and carries
+// `uint64_t* stamps` makes the kernel record, per workgroup, the shader-clock counter and the
+// constant-rate counter at four points: start, first stage landed, main loop done, epilogue done
+// (stamps[8 * workgroup + 2 * point + {0, 1}]).
+template <typename E, typename = void>
+struct epi_profiled : std::false_type {};
+template <typename E>
+struct epi_profiled<E, typename std::enable_if<E::PROFILED>::type> : std::true_type {};
+template <typename Epi>
+struct EpiProfiled : Epi {
+  uint64_t* stamps;
+  static constexpr bool PROFILED = true;
+};
+
 // The epilogue of K range `split` (blockIdx.y): only the partial store depends on it.
 template <typename Epi>
 __device__ __forceinline__ Epi epilogue_of_split(const Epi& e, int) { return e; }
@@ -399,6 +413,16 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   const int l = t & 63;
   const int w = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wm = w >> 1, wn = w & 1;
+  auto stamp = [&](int point) {
+    if constexpr (epi_profiled<Epi>::value) {
+      if (threadIdx.x == 0) {
+        uint64_t* p = epi.stamps + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 8 + 2 * point;
+        p[0] = __builtin_amdgcn_s_memtime();
+        p[1] = __builtin_amdgcn_s_memrealtime();
+      }
+    }
+  };
+  stamp(0);
 
   int tm, tn;
   tile_of_workgroup(tiles_m, tiles_n, tm, tn);
@@ -490,30 +514,33 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   auto dma_piece = [&](int st, int slot, int pslot, int d, auto steady_const) {
     constexpr bool STEADY = decltype(steady_const)::value;
     if (!STEADY) st = st < KTS ? st : KTS - 1;
-    const bool part_pair = !STEADY && pair_valid < 8 && (st >> 1) == last_pair;
+    // (no branches here: the instruction order of a stage is pinned slot by slot)
+    const bool last_pair_now = !STEADY && (st >> 1) == last_pair;
     if (d < DMA_B) {
       const int q = DMA_B * w + d;
       if (BPAIR) {
         const uint32_t dst = lds_base + slot * BPAIR_BYTES + PairDma::dma_lds(q >> 1, q & 1);
-        if (part_pair)
-          dma16z(b_tile + (int64_t)(st >> 1) * 128, b_voff[d], dst, pair_piece(q) >= pair_valid);
-        else
+        if (STEADY)
           dma16(b_tile + (int64_t)(st >> 1) * 128, b_voff[d], dst);
+        else
+          dma16z(b_tile + (int64_t)(st >> 1) * 128, b_voff[d], dst,
+                 last_pair_now && pair_piece(q) >= pair_valid);
       } else {
         const uint32_t dst = lds_base + slot * OPERAND_BYTES + BT::dma_lds(q >> 2, q & 3);
-        if (!STEADY && tail_k < KB && st == KTS - 1)
-          dma16z(b_tile + (int64_t)st * b_kstep, b_voff[d], dst,
-                 BT::dma_k(q >> 2, q & 3, l) * Math::ELEM_BYTES >= tail_k);
-        else
+        if (STEADY)
           dma16(b_tile + (int64_t)st * b_kstep, b_voff[d], dst);
+        else
+          dma16z(b_tile + (int64_t)st * b_kstep, b_voff[d], dst,
+                 st == KTS - 1 && BT::dma_k(q >> 2, q & 3, l) * Math::ELEM_BYTES >= tail_k);
       }
     } else {
       const int q = DMA_A * w + d - DMA_B;
       const uint32_t dst = lds_base + B_RING + pslot * APAIR_BYTES + PairDma::dma_lds(q >> 1, q & 1);
-      if (part_pair)
-        dma16z(a_tile + (int64_t)(st >> 1) * 128, a_voff[d - DMA_B], dst, pair_piece(q) >= pair_valid);
-      else
+      if (STEADY)
         dma16(a_tile + (int64_t)(st >> 1) * 128, a_voff[d - DMA_B], dst);
+      else
+        dma16z(a_tile + (int64_t)(st >> 1) * 128, a_voff[d - DMA_B], dst,
+               last_pair_now && pair_piece(q) >= pair_valid);
     }
   };
   typedef std::integral_constant<bool, true> steady_t;
@@ -593,6 +620,7 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int r = 0; r < NREAD; ++r) read_piece(f0, 0, 0, 0, 0, r);
+  stamp(1);
   // Single B stages: ring slots of the stage being multiplied, of the next one, and of the one
   // the DMA fills (wave-uniform scalars, advanced modulo NSTAGES each stage).  B pairs: the
   // slot of the pair being multiplied and the other one, swapped every second stage; the DMA
@@ -693,6 +721,7 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   if (KTS & 1) stage(KTS - 1, std::integral_constant<int, 0>{}, drain_t{});
   wait_vmcnt(std::integral_constant<int, 0>{});  // no DMA outlives the main loop
   __syncthreads();  // ... for any wave, and every wave is done reading the ring
+  stamp(2);
 
   // ---- epilogue -----------------------------------------------------------------------------
   // acc[i][j][4q+e] = C[m0 + wm*32*MT + 32i + l%32][n0 + wn*128 + 32j + 8q + 4g + e]: a lane
@@ -738,6 +767,16 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
         colv[j][q] = epi.load_cols(col < N ? col : N - 4);
       }
   }
+  // Store side of the staging: lane -> (row within a pass, 16-byte piece of the 128-column row).
+  // N is a multiple of 4: a piece of 32-bit outputs is in or out as a whole, one of 16-bit
+  // outputs may be half inside (then its first 8 bytes are stored).
+  constexpr int NPASS = 32 / ROWS_PER_PASS;
+  const int lane_row = le / LANES_PER_ROW, c16 = le % LANES_PER_ROW;
+  const int64_t piece_col = n0 + wn * 128 + c16 * (16 / OB);
+  const bool piece_in = piece_col < N;
+  const bool piece_half = OB == 2 && piece_col + 8 > N;
+  const int64_t row_step = (intptr_t)epi.out_row(1) - (intptr_t)epi.out_row(0);  // bytes per row
+  const bool interior = m0 + TILE_M <= M && n0 + BN <= N;  // (uniform)
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     const int64_t row0 = m0 + wm * 32 * MT + 32 * i;
@@ -763,23 +802,39 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
           epi.side(row, col, acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
                    acc[i][j][4 * q + 3]);
       }
+    // All pieces of the block are read back into registers first and then stored: one LDS
+    // latency per row tile instead of one per store instruction.  Row addresses advance by a
+    // constant; the bounds checks exist only in workgroups on the matrix edge.
+    u32x4 v[NPASS];
 #pragma unroll
-    for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
-      const int rl = p * ROWS_PER_PASS + le / LANES_PER_ROW;
-      const int c16 = le % LANES_PER_ROW;
-      const u32x4 v = *reinterpret_cast<const u32x4*>(scr + rl * ROW_STRIDE + c16 * 16);
-      // N is a multiple of 4: a 16-byte piece of 32-bit outputs is in or out as a whole, one
-      // of 16-bit outputs may be half inside (then its first 8 bytes are stored)
-      const int64_t piece_col = n0 + wn * 128 + c16 * (16 / OB);
-      if (row0 + rl < M && piece_col < N) {
-        char* dst = epi.out_row(row0 + rl) + (n0 + wn * 128) * OB + c16 * 16;
+    for (int p = 0; p < NPASS; ++p)
+      v[p] = *reinterpret_cast<const u32x4*>(scr + (p * ROWS_PER_PASS + lane_row) * ROW_STRIDE +
+                                             c16 * 16);
+    __builtin_amdgcn_sched_barrier(0);
+    char* dst0 = epi.out_row(row0 + lane_row) + (n0 + wn * 128) * OB + c16 * 16;
+    if (interior) {
+#pragma unroll
+      for (int p = 0; p < NPASS; ++p)
         // streaming stores: C is not read again by this kernel and should not evict A / B
-        if (OB == 2 && piece_col + 8 > N)
-          __builtin_nontemporal_store(u32x2{v[0], v[1]}, reinterpret_cast<u32x2*>(dst));
-        else
-          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
+        __builtin_nontemporal_store(v[p],
+                                    reinterpret_cast<u32x4*>(dst0 + p * ROWS_PER_PASS * row_step));
+    } else {
+#pragma unroll
+      for (int p = 0; p < NPASS; ++p) {
+        char* dst = dst0 + p * ROWS_PER_PASS * row_step;
+        if (row0 + p * ROWS_PER_PASS + lane_row < M && piece_in) {
+          if (piece_half)
+            __builtin_nontemporal_store(u32x2{v[p][0], v[p][1]}, reinterpret_cast<u32x2*>(dst));
+          else
+            __builtin_nontemporal_store(v[p], reinterpret_cast<u32x4*>(dst));
+        }
       }
     }
+  }
+  if constexpr (epi_profiled<Epi>::value) {
+    // the epilogue ends when this wave's stores have been acknowledged
+    wait_vmcnt(std::integral_constant<int, 0>{});
+    stamp(3);
   }
 }
 

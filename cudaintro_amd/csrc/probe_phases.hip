@@ -1,0 +1,87 @@
+// Measurement aid: one launch of the 256-row, four-wave LDS-tiled matrix-core kernel with
+// timestamps taken inside every workgroup (start, first stage landed, main loop done, stores
+// acknowledged), reduced on the host to the time each phase takes, the matrix-core issue cycles
+// per stage and the shader clock the chip held in the main loop.  The kernel is the product
+// kernel itself (same template, same schedule); only the four stamps are added.
+#include <algorithm>
+#include <vector>
+
+#include "epilogues.h"
+#include "mfma_tile.h"
+
+namespace cig {
+namespace {
+
+template <typename Math, int BMODE, typename Epi>
+cigemmStatus_t run_profiled(cigemmContext* ctx, const char* name, int64_t M, int64_t N,
+                            int64_t K_bytes, const void* A, int64_t lda_bytes, const void* B,
+                            int64_t ldb_bytes, const Epi& base, double* out) {
+  const int64_t tiles = ((M + 255) / 256) * ((N + tile::BN - 1) / tile::BN);
+  if (!ctx->workspace || (size_t)tiles * 64 > ctx->ws_partial_bytes)
+    return fail(ctx, CIGEMM_STATUS_NOT_SUPPORTED, "%s: %lld tiles exceed the workspace", name,
+                (long long)tiles);
+  uint64_t* stamps = static_cast<uint64_t*>(ctx->workspace);
+  tile::EpiProfiled<Epi> epi{base, stamps};
+  tile::launch_tile_mt<Math, BMODE, 4, tile::EpiProfiled<Epi>, 2>(ctx, M, N, K_bytes, A, lda_bytes,
+                                                                 B, ldb_bytes, epi);
+  cigemmStatus_t st = check_launch(ctx, name);
+  if (st != CIGEMM_STATUS_SUCCESS) return st;
+  std::vector<uint64_t> h((size_t)tiles * 8);
+  if (hipMemcpyAsync(h.data(), stamps, h.size() * 8, hipMemcpyDeviceToHost, ctx->stream) != hipSuccess ||
+      hipStreamSynchronize(ctx->stream) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(ctx, CIGEMM_STATUS_EXECUTION_FAILED, "%s: reading the stamps back failed", name);
+  }
+  // constant-rate counter: 100 MHz on this chip (10 ns per tick)
+  const double tick_us = 0.01;
+  const int64_t kts = (K_bytes + tile::KB - 1) / tile::KB;
+  double phase_us[3] = {0, 0, 0}, main_cycles = 0, main_ticks = 0;
+  uint64_t first_start = ~0ull, last_end = 0, first_epi = ~0ull, last_main_end = 0;
+  for (int64_t g = 0; g < tiles; ++g) {
+    const uint64_t* s = &h[(size_t)g * 8];
+    for (int p = 0; p < 3; ++p) phase_us[p] += (double)(s[2 * p + 3] - s[2 * p + 1]) * tick_us;
+    main_cycles += (double)(s[4] - s[2]);
+    main_ticks += (double)(s[5] - s[3]);
+    first_start = std::min(first_start, s[1]);
+    last_end = std::max(last_end, s[7]);
+    first_epi = std::min(first_epi, s[5]);
+    last_main_end = std::max(last_main_end, s[5]);
+  }
+  out[0] = phase_us[0] / tiles;                       // start -> first stage in registers
+  out[1] = phase_us[1] / tiles;                       // main loop
+  out[2] = phase_us[2] / tiles;                       // epilogue, stores acknowledged
+  out[3] = (double)(last_end - first_start) * tick_us;  // first workgroup start -> last end
+  out[4] = main_cycles / tiles / (double)kts;         // shader cycles per 64-byte stage
+  out[5] = main_cycles / (main_ticks * tick_us) * 1e-3;  // GHz held in the main loop
+  out[6] = (double)(last_end - first_epi) * tick_us;  // first epilogue start -> last end
+  out[7] = (double)tiles;
+  ctx->last_kernel = "tile_phase_probe";
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+}  // namespace
+}  // namespace cig
+
+using namespace cig;
+
+extern "C" cigemmStatus_t cigemm_probe_tile_phases(cigemmHandle_t h, int kind, int64_t M,
+                                                   int64_t N, int64_t K, const void* A,
+                                                   int64_t lda, const void* B, int64_t ldb,
+                                                   void* C, int64_t ldc, double* phases) {
+  const char* name = "cigemm_probe_tile_phases";
+  if (!h || h->magic != kCtxMagic) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if (kind < 0 || kind > 1 || !A || !B || !C || !phases || M <= 0 || N <= 0 || K <= 0 ||
+      lda < K || ldb < N || ldc < N)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: bad argument", name);
+  const int elem = kind == 0 ? 2 : 1;
+  if (!tile::tile_shape_ok(M, N, K, elem, A, lda, B, ldb, true) || N % 8 || ldc % 8 ||
+      ((uintptr_t)C & 15))
+    return fail(h, CIGEMM_STATUS_NOT_SUPPORTED, "%s: shape or alignment outside the tile kernel's",
+                name);
+  if (kind == 0)
+    return run_profiled<tile::MathBF16, tile::B_KN16>(h, name, M, N, K * 2, A, lda * 2, B, ldb * 2,
+                                                      EpiStore16x4<BF16>{static_cast<uint16_t*>(C), ldc},
+                                                      phases);
+  return run_profiled<tile::MathI8, tile::B_KN8>(h, name, M, N, K, A, lda, B, ldb,
+                                                 EpiStoreI32x4{static_cast<int32_t*>(C), ldc}, phases);
+}

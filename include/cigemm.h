@@ -78,7 +78,14 @@ CIGEMM_API cigemmStatus_t cigemmCreate(cigemmHandle_t* handle);
 CIGEMM_API cigemmStatus_t cigemmDestroy(cigemmHandle_t handle);
 
 /* Replaces cublasSetStream (implicit default stream in the reference).  `stream` is a
- * hipStream_t passed as void*; NULL selects the null stream. */
+ * hipStream_t passed as void*; NULL selects the null stream.
+ * The handle owns ONE workspace (64 MiB of split-K partial sums plus arrival counters,
+ * allocated by cigemmCreate) that every split-K call on it uses.  Calls on one handle must
+ * therefore not overlap on the device: switching the handle to another stream while work
+ * enqueued on the old one may still be running, or replaying a captured graph concurrently
+ * with eager calls on the same handle, races on that workspace and gives wrong results
+ * without an error.  Order the streams yourself (an event) before switching, or use one
+ * handle per stream. */
 CIGEMM_API cigemmStatus_t cigemmSetStream(cigemmHandle_t handle, void* stream);
 CIGEMM_API cigemmStatus_t cigemmGetStream(cigemmHandle_t handle, void** stream);
 
@@ -237,11 +244,32 @@ CIGEMM_API cigemmStatus_t cigemm_matrixMulMatrixCoresBfloat16(cigemmHandle_t han
 CIGEMM_API cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t handle, int kind, int random_bits,
                                             int iters, int64_t* ops_per_launch);
 
+/* No counterpart in the reference.  Runs ONE launch of the 256-row, four-wave LDS-tiled
+ * matrix-core kernel (the product kernel with four timestamps added per workgroup) on the
+ * handle's stream, waits for it, and reduces the stamps: kind 0 = bf16 (A, B, C as in
+ * cigemm_gemm_bf16), 1 = int8 K x N operands, int32 out (as cigemm_gemm_i8_i32 with
+ * CIGEMM_B_KN).  Same shape and alignment conditions as the tile kernel, N % 8 == 0.
+ * phases[0..7] receive, averaged over the workgroups: microseconds from workgroup start to the
+ * first stage in registers; of the main loop; of the epilogue until its stores are
+ * acknowledged; microseconds from the first workgroup's start to the last one's end; shader
+ * cycles per 64-byte stage of k in the main loop; shader clock (GHz) held in the main loop;
+ * microseconds from the first workgroup entering its epilogue to the last one's end; number of
+ * workgroups.  Synchronises the stream; meant for profiling runs, not for the hot path. */
+CIGEMM_API cigemmStatus_t cigemm_probe_tile_phases(cigemmHandle_t handle, int kind, int64_t M,
+                                                   int64_t N, int64_t K, const void* A,
+                                                   int64_t lda, const void* B, int64_t ldb,
+                                                   void* C, int64_t ldc, double* phases);
+
 /* ---- device-side input generation -------------------------------------------------- */
 
 /* Replace fill_random_fp32 / _bf16 / _fp16 / _int8 (quantization/GEMM_fp32.cu:7-17,
  * GEMM_bf16.cu:8-19, GEMM_fp16.cu:8-19, GEMM_int8.cu:8-19): element idx gets the value
- * derived from ((idx ^ seed) * 2862933555777941757 + 3037000493) mod 2^64. */
+ * derived from ((idx ^ seed) * 2862933555777941757 + 3037000493) mod 2^64.
+ * The affine map lo + r * (hi - lo) is evaluated as a separately rounded multiply and add.
+ * The reference's build (plain nvcc -O3) may contract it into one fused multiply-add; the two
+ * agree bit for bit whenever r * (hi - lo) is exact in fp32, which holds for the suite's own
+ * range lo = -1, hi = 1 (the case the known-answer vectors pin).  For other ranges parity
+ * with the reference's generator is not pinned. */
 CIGEMM_API cigemmStatus_t cigemm_fill_random_f32(cigemmHandle_t handle, float* data,
                                                  int64_t count, uint64_t seed, float lo,
                                                  float hi);
