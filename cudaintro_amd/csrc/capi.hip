@@ -42,10 +42,10 @@ void set_tile_kernel_name(cigemmContext* ctx, const char* dtype, int k_elems, co
     snprintf(waves, sizeof(waves), "w%d+w%d", ctx->first_waves, ctx->last_waves);
   } else {
     snprintf(rows, sizeof(rows), "%d", ctx->last_tile_rows);
-    snprintf(waves, sizeof(waves), "w%d", ctx->last_waves);
+    snprintf(waves, sizeof(waves), ctx->last_per_cu == 2 ? "w%dx2" : "w%d", ctx->last_waves);
   }
-  snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_mfma_%sx256x%d_%s_ring4%s%s", dtype,
-           rows, k_elems, waves, suffix, splitk ? "_splitk" : "");
+  snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_mfma_%sx256x%d_%s_ring%d%s%s", dtype,
+           rows, k_elems, waves, ctx->last_per_cu == 2 ? 3 : 4, suffix, splitk ? "_splitk" : "");
   ctx->last_kernel = ctx->kernel_name;
 }
 
@@ -75,6 +75,7 @@ cigemmStatus_t check_gemm_args(cigemmHandle_t h, const char* name, int64_t M, in
   h->last_tile_rows = 0;  // set again by the tile kernel's launcher
   h->last_k_splits = 0;
   h->last_waves = 0;
+  h->last_per_cu = 1;
   h->first_tile_rows = 0;
   h->first_waves = 0;
   if (M < 0 || N < 0 || K < 0)
@@ -133,6 +134,11 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->last_tile_rows = 0;
   ctx->last_k_splits = 0;
   ctx->last_waves = 0;
+  ctx->last_per_cu = 1;
+  {
+    const char* e = getenv("CIGEMM_TILE2");   // experiment switch: 0 = never, 1 = always
+    ctx->tile2_mode = e ? atoi(e) : 0;
+  }
   ctx->first_tile_rows = 0;
   ctx->first_waves = 0;
   ctx->kernel_name[0] = '\0';

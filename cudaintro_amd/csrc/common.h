@@ -20,6 +20,8 @@ struct cigemmContext {
   int last_tile_rows;  // rows of the output tile of the last tile-kernel launch, 0 otherwise
   int last_k_splits;   // K ranges of that launch
   int last_waves;      // wavefronts per workgroup of that launch
+  int last_per_cu;     // workgroups of that launch resident per compute unit (1 or 2)
+  int tile2_mode;      // which shapes take the two-workgroups-per-unit tile kernel (see capi.hip)
   int first_tile_rows; // when the call took two launches: rows and waves of the first, else 0
   int first_waves;
   char kernel_name[96];  // storage for names composed per call (last_kernel may point here)

@@ -371,6 +371,122 @@ __device__ __forceinline__ EpiPartialX4 epilogue_of_split(const EpiPartialX4& e,
   return EpiPartialX4{e.base + split * e.split_stride, e.ld, e.split_stride};
 }
 
+// The epilogue of the tile kernels: accumulators -> output rows.
+// acc[i][j][4q+e] = C[m0 + wm*32*MT + 32i + l%32][n0 + wn*128 + 32j + 8q + 4g + e]: a lane
+// holds short pieces of 32 different rows.  Each wave stages one 32-row x 128-column block
+// at a time in its own piece of the (now idle) LDS and writes it out as whole rows: every
+// store instruction then covers full 256- or 512-byte row segments.  Call it once every wave
+// of the workgroup has stopped reading the operand ring and no DMA is in flight.
+template <typename Math, int MT, int NW, int TILE_M, typename Epi>
+__device__ __forceinline__ void store_tile(const Epi& epi, typename Math::acc_t (&acc)[MT][4],
+                                           char* lds, int w, int wm, int wn, int64_t m0,
+                                           int64_t n0, int M, int N, float epi_row_word,
+                                           float epi_col_word) {
+  // The epilogue takes the lane number afresh from the hardware (and opaque to the compiler),
+  // so that neither it nor any of the epilogue's addresses is held in a register through the
+  // main loop.
+  int le = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  asm volatile("" : "+v"(le));
+  le &= 63;
+  const int ge = le >> 5;
+  constexpr int OB = Epi::OUT_BYTES;
+  constexpr int ROW_BYTES = 128 * OB;
+  constexpr int ROW_STRIDE = ROW_BYTES + 16;
+  constexpr int LANES_PER_ROW = ROW_BYTES / 16;
+  constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+  // (the launcher sizes the dynamic LDS for the larger of the ring and these staging blocks)
+  static_assert(NW * 32 * ROW_STRIDE <= 160 * 1024, "the waves' staging blocks must fit the LDS");
+  char* scr = lds + w * (32 * ROW_STRIDE);
+  typedef decltype(epi.pack((int64_t)0, (int64_t)0, acc[0][0][0], acc[0][0][0], acc[0][0][0],
+                            acc[0][0][0])) packed_t;
+  // What the epilogue needs per column quad (scales, bias) is the same for every row tile:
+  // fetched once, up front, so that no load latency sits between the accumulator reads.
+  typename Epi::col_t colv[4][4];
+  bool cols_done = false;
+  if constexpr (epi_has_uniform_mode<Epi>::value) {
+    if (epi.col_uniform()) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) colv[j][q] = epi.cols_from_word(epi_col_word);
+      cols_done = true;
+    }
+  }
+  if (!cols_done) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t col = n0 + wn * 128 + 32 * j + 8 * q + 4 * ge;
+        colv[j][q] = epi.load_cols(col < N ? col : N - 4);
+      }
+  }
+  // Store side of the staging: lane -> (row within a pass, 16-byte piece of the 128-column row).
+  // N is a multiple of 4: a piece of 32-bit outputs is in or out as a whole, one of 16-bit
+  // outputs may be half inside (then its first 8 bytes are stored).
+  constexpr int NPASS = 32 / ROWS_PER_PASS;
+  const int lane_row = le / LANES_PER_ROW, c16 = le % LANES_PER_ROW;
+  const int64_t piece_col = n0 + wn * 128 + c16 * (16 / OB);
+  const bool piece_in = piece_col < N;
+  const bool piece_half = OB == 2 && piece_col + 8 > N;
+  const int64_t row_step = (intptr_t)epi.out_row(1) - (intptr_t)epi.out_row(0);  // bytes per row
+  const bool interior = m0 + TILE_M <= M && n0 + BN <= N;  // (uniform)
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const int64_t row0 = m0 + wm * 32 * MT + 32 * i;
+    const int64_t row = row0 + (le & 31);
+    const bool row_ok = row < M;
+    const int64_t row_c = row_ok ? row : M - 1;  // scale lookups stay in bounds
+    typename Epi::row_t rowv;
+    if constexpr (epi_has_uniform_mode<Epi>::value)
+      rowv = epi.row_uniform() ? epi.row_from_word(epi_row_word) : epi.load_row(row_c);
+    else
+      rowv = epi.load_row(row_c);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int c = 32 * j + 8 * q + 4 * ge;
+        const int64_t col = n0 + wn * 128 + c;
+        const bool col_ok = col < N;  // N is a multiple of 4: a quad is in or out as a whole
+        *reinterpret_cast<packed_t*>(scr + (le & 31) * ROW_STRIDE + c * OB) =
+            epi.pack(rowv, colv[j][q], acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
+                     acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        if (row_ok && col_ok)
+          epi.side(row, col, acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                   acc[i][j][4 * q + 3]);
+      }
+    // All pieces of the block are read back into registers first and then stored: one LDS
+    // latency per row tile instead of one per store instruction.  Row addresses advance by a
+    // constant; the bounds checks exist only in workgroups on the matrix edge.
+    u32x4 v[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p)
+      v[p] = *reinterpret_cast<const u32x4*>(scr + (p * ROWS_PER_PASS + lane_row) * ROW_STRIDE +
+                                             c16 * 16);
+    __builtin_amdgcn_sched_barrier(0);
+    char* dst0 = epi.out_row(row0 + lane_row) + (n0 + wn * 128) * OB + c16 * 16;
+    if (interior) {
+#pragma unroll
+      for (int p = 0; p < NPASS; ++p)
+        // streaming stores: C is not read again by this kernel and should not evict A / B
+        __builtin_nontemporal_store(v[p],
+                                    reinterpret_cast<u32x4*>(dst0 + p * ROWS_PER_PASS * row_step));
+    } else {
+#pragma unroll
+      for (int p = 0; p < NPASS; ++p) {
+        char* dst = dst0 + p * ROWS_PER_PASS * row_step;
+        if (row0 + p * ROWS_PER_PASS + lane_row < M && piece_in) {
+          if (piece_half)
+            __builtin_nontemporal_store(u32x2{v[p][0], v[p][1]}, reinterpret_cast<u32x2*>(dst));
+          else
+            __builtin_nontemporal_store(v[p], reinterpret_cast<u32x4*>(dst));
+        }
+      }
+    }
+  }
+}
+
 // Epi: an epilogue functor (see epilogues.h): load_row / load_cols / pack / side / out_row.
 //
 // A, B are byte pointers; lda/ldb are in BYTES.  Any M; N a multiple of 4; all rows 16-byte
@@ -724,113 +840,8 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   stamp(2);
 
   // ---- epilogue -----------------------------------------------------------------------------
-  // acc[i][j][4q+e] = C[m0 + wm*32*MT + 32i + l%32][n0 + wn*128 + 32j + 8q + 4g + e]: a lane
-  // holds short pieces of 32 different rows.  Each wave stages one 32-row x 128-column block
-  // at a time in its own piece of the (now idle) LDS and writes it out as whole rows: every
-  // store instruction then covers full 256- or 512-byte row segments.
-  // The epilogue takes the lane number afresh from the hardware (and opaque to the compiler),
-  // so that neither it nor any of the epilogue's addresses is held in a register through the
-  // main loop.
-  int le = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-  asm volatile("" : "+v"(le));
-  le &= 63;
-  const int ge = le >> 5;
-  constexpr int OB = Epi::OUT_BYTES;
-  constexpr int ROW_BYTES = 128 * OB;
-  constexpr int ROW_STRIDE = ROW_BYTES + 16;
-  constexpr int LANES_PER_ROW = ROW_BYTES / 16;
-  constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
-  // (the launcher sizes the dynamic LDS for the larger of the ring and these staging blocks)
-  static_assert(NW * 32 * ROW_STRIDE <= 160 * 1024, "the waves' staging blocks must fit the LDS");
-  char* scr = lds + w * (32 * ROW_STRIDE);
-  typedef decltype(epi.pack((int64_t)0, (int64_t)0, acc[0][0][0], acc[0][0][0], acc[0][0][0],
-                            acc[0][0][0])) packed_t;
-  // What the epilogue needs per column quad (scales, bias) is the same for every row tile:
-  // fetched once, up front, so that no load latency sits between the accumulator reads.
-  typename Epi::col_t colv[4][4];
-  bool cols_done = false;
-  if constexpr (epi_has_uniform_mode<Epi>::value) {
-    if (epi.col_uniform()) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) colv[j][q] = epi.cols_from_word(epi_col_word);
-      cols_done = true;
-    }
-  }
-  if (!cols_done) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int64_t col = n0 + wn * 128 + 32 * j + 8 * q + 4 * ge;
-        colv[j][q] = epi.load_cols(col < N ? col : N - 4);
-      }
-  }
-  // Store side of the staging: lane -> (row within a pass, 16-byte piece of the 128-column row).
-  // N is a multiple of 4: a piece of 32-bit outputs is in or out as a whole, one of 16-bit
-  // outputs may be half inside (then its first 8 bytes are stored).
-  constexpr int NPASS = 32 / ROWS_PER_PASS;
-  const int lane_row = le / LANES_PER_ROW, c16 = le % LANES_PER_ROW;
-  const int64_t piece_col = n0 + wn * 128 + c16 * (16 / OB);
-  const bool piece_in = piece_col < N;
-  const bool piece_half = OB == 2 && piece_col + 8 > N;
-  const int64_t row_step = (intptr_t)epi.out_row(1) - (intptr_t)epi.out_row(0);  // bytes per row
-  const bool interior = m0 + TILE_M <= M && n0 + BN <= N;  // (uniform)
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    const int64_t row0 = m0 + wm * 32 * MT + 32 * i;
-    const int64_t row = row0 + (le & 31);
-    const bool row_ok = row < M;
-    const int64_t row_c = row_ok ? row : M - 1;  // scale lookups stay in bounds
-    typename Epi::row_t rowv;
-    if constexpr (epi_has_uniform_mode<Epi>::value)
-      rowv = epi.row_uniform() ? epi.row_from_word(epi_row_word) : epi.load_row(row_c);
-    else
-      rowv = epi.load_row(row_c);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int c = 32 * j + 8 * q + 4 * ge;
-        const int64_t col = n0 + wn * 128 + c;
-        const bool col_ok = col < N;  // N is a multiple of 4: a quad is in or out as a whole
-        *reinterpret_cast<packed_t*>(scr + (le & 31) * ROW_STRIDE + c * OB) =
-            epi.pack(rowv, colv[j][q], acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
-                     acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-        if (row_ok && col_ok)
-          epi.side(row, col, acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                   acc[i][j][4 * q + 3]);
-      }
-    // All pieces of the block are read back into registers first and then stored: one LDS
-    // latency per row tile instead of one per store instruction.  Row addresses advance by a
-    // constant; the bounds checks exist only in workgroups on the matrix edge.
-    u32x4 v[NPASS];
-#pragma unroll
-    for (int p = 0; p < NPASS; ++p)
-      v[p] = *reinterpret_cast<const u32x4*>(scr + (p * ROWS_PER_PASS + lane_row) * ROW_STRIDE +
-                                             c16 * 16);
-    __builtin_amdgcn_sched_barrier(0);
-    char* dst0 = epi.out_row(row0 + lane_row) + (n0 + wn * 128) * OB + c16 * 16;
-    if (interior) {
-#pragma unroll
-      for (int p = 0; p < NPASS; ++p)
-        // streaming stores: C is not read again by this kernel and should not evict A / B
-        __builtin_nontemporal_store(v[p],
-                                    reinterpret_cast<u32x4*>(dst0 + p * ROWS_PER_PASS * row_step));
-    } else {
-#pragma unroll
-      for (int p = 0; p < NPASS; ++p) {
-        char* dst = dst0 + p * ROWS_PER_PASS * row_step;
-        if (row0 + p * ROWS_PER_PASS + lane_row < M && piece_in) {
-          if (piece_half)
-            __builtin_nontemporal_store(u32x2{v[p][0], v[p][1]}, reinterpret_cast<u32x2*>(dst));
-          else
-            __builtin_nontemporal_store(v[p], reinterpret_cast<u32x4*>(dst));
-        }
-      }
-    }
-  }
+  store_tile<Math, MT, NW, TILE_M>(epi, acc, lds, w, wm, wn, m0, n0, M, N, epi_row_word,
+                                   epi_col_word);
   if constexpr (epi_profiled<Epi>::value) {
     // the epilogue ends when this wave's stores have been acknowledged
     wait_vmcnt(std::integral_constant<int, 0>{});
@@ -856,6 +867,7 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
   ctx->last_tile_rows = TILE_M;
   ctx->last_k_splits = splits;
   ctx->last_waves = 2 * WM;
+  ctx->last_per_cu = 1;
   // stages per K range; only an unsplit K may leave its last stage partly filled
   const int64_t kts = splits > 1 ? K_bytes / KB / splits : (K_bytes + KB - 1) / KB;
   const int64_t range_bytes = splits > 1 ? kts * KB : K_bytes;
