@@ -360,6 +360,27 @@ def main():
         log(f"[bench] fp16 {n}^3")
         per_config[f"fp16_{n}"] = run16("f16")
 
+        # The same headline problem on the two-workgroups-per-unit form of the tile kernel
+        # (CIGEMM_ALGO_TILE_PAIRED, never chosen by default): more matrix instructions issued
+        # per cycle, a lower clock under the power limit.  Recorded as the measured reason for
+        # the default's choice.
+        a_b, b_b = wl.normal_16bit(n, n, n, seed=2, kind="bf16")
+        a, b = dev16(torch, a_b, "bf16"), dev16(torch, b_b, "bf16")
+        c = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
+        with handle.algo(ci.ALGO_TILE_PAIRED):
+            w, e = time_calls(torch, lambda: handle.gemm_bf16(a, b, out=c), args.steps, args.warmup)
+            name_p = handle.last_kernel
+        t = ops * args.steps / e / 1e12
+        for _ in range(3):
+            ph = handle.probe_tile_phases(a, b, c, paired=True)
+        per_config[f"bf16_{n}_two_workgroups_per_unit"] = {
+            "tflops": t, "frac_of_peak": t / PEAK_16BIT_TFLOPS, "peak": PEAK_16BIT_TFLOPS,
+            "ms": e / args.steps * 1e3, "ms_over_default": e / args.steps / (ev / args.steps),
+            "kernel": name_p, "phases": ph,
+            # two workgroups share a unit's matrix cores: 2 x 512 issue cycles per stage pair
+            "mfma_issue_fraction_of_main_loop": 1024.0 / ph["cycles_per_stage"]}
+        del a, b, c
+
         # shapes that do not fill the kernel's units: a K whose last 64-byte stage holds one
         # 16-byte piece, an N whose last column tile holds 8 columns (no alignment cliff wanted)
         for (Mx, Nx, Kx) in ((n, n, n + 8), (n, n + 8, n)):

@@ -14,6 +14,7 @@ from .cigemm import (  # noqa: F401
     ALGO_SKINNY,
     ALGO_SMALL,
     ALGO_TILE,
+    ALGO_TILE_PAIRED,
     B_KN,
     B_NK,
     OUT_BF16,

@@ -17,7 +17,7 @@ _SUITE = os.path.join(_HERE, "gemm_suite")
 
 B_KN, B_NK = 0, 1
 ACT_NONE, ACT_RELU = 0, 1
-ALGO_DEFAULT, ALGO_GENERIC, ALGO_TILE, ALGO_SKINNY, ALGO_SMALL = -1, 0, 1, 2, 3
+ALGO_DEFAULT, ALGO_GENERIC, ALGO_TILE, ALGO_SKINNY, ALGO_SMALL, ALGO_TILE_PAIRED = -1, 0, 1, 2, 3, 4
 SCALE_TENSOR, SCALE_VECTOR = 0, 1
 OUT_F32, OUT_BF16 = 0, 1
 
@@ -271,11 +271,12 @@ class Handle:
                     "cigemm_probe_mfma")
         return ops.value
 
-    def probe_tile_phases(self, A, B, out):
-        """One instrumented launch of the 256-row tile kernel (bf16 or int8 K x N -> int32);
-        returns the phase figures as a dict (see cigemm_probe_tile_phases)."""
+    def probe_tile_phases(self, A, B, out, paired=False):
+        """One instrumented launch of the 256-row tile kernel, or with ``paired`` of its
+        two-workgroups-per-unit form (bf16 or int8 K x N -> int32); returns the phase figures
+        as a dict (see cigemm_probe_tile_phases)."""
         torch = _torch()
-        kind = {torch.bfloat16: 0, torch.int8: 1}[A.dtype]
+        kind = {torch.bfloat16: 0, torch.int8: 1}[A.dtype] + (2 if paired else 0)
         M, K = A.shape
         N = B.shape[1]
         ph = (C.c_double * 8)()

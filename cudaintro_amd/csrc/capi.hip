@@ -135,10 +135,6 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->last_k_splits = 0;
   ctx->last_waves = 0;
   ctx->last_per_cu = 1;
-  {
-    const char* e = getenv("CIGEMM_TILE2");   // experiment switch: 0 = never, 1 = always
-    ctx->tile2_mode = e ? atoi(e) : 0;
-  }
   ctx->first_tile_rows = 0;
   ctx->first_waves = 0;
   ctx->kernel_name[0] = '\0';
@@ -212,7 +208,7 @@ cigemmStatus_t cigemmGetLastPlan(cigemmHandle_t h, int* tile_rows, int* k_splits
 
 cigemmStatus_t cigemmSetAlgo(cigemmHandle_t h, cigemmAlgo_t algo) {
   if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
-  if ((int)algo < CIGEMM_ALGO_DEFAULT || (int)algo > CIGEMM_ALGO_SMALL)
+  if ((int)algo < CIGEMM_ALGO_DEFAULT || (int)algo > CIGEMM_ALGO_TILE_PAIRED)
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "cigemmSetAlgo: bad algo %d", (int)algo);
   h->algo = (int)algo;
   return CIGEMM_STATUS_SUCCESS;
@@ -243,6 +239,7 @@ static bool dispatch_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K, cons
       launch_f32_small(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
       return true;
     case CIGEMM_ALGO_SKINNY:
+    case CIGEMM_ALGO_TILE_PAIRED:
       return false;
     case CIGEMM_ALGO_GENERIC:
       launch_generic_f32(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
@@ -288,6 +285,9 @@ static cigemmStatus_t gemm16(cigemmHandle_t h, const char* name, bool bf16, int6
   switch (h->algo) {
     case CIGEMM_ALGO_SKINNY: ok = launch_skinny_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
     case CIGEMM_ALGO_TILE: ok = launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
+    case CIGEMM_ALGO_TILE_PAIRED:
+      ok = launch_16b_mfma_paired(h, bf16, M, N, K, A, lda, B, ldb, C, ldc);
+      break;
     case CIGEMM_ALGO_SMALL: ok = false; break;
     case CIGEMM_ALGO_GENERIC: launch_generic_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
     default:
@@ -321,6 +321,9 @@ static cigemmStatus_t gemm_i8(cigemmHandle_t h, const char* name, int64_t M, int
   switch (h->algo) {
     case CIGEMM_ALGO_SKINNY: ok = launch_skinny_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq); break;
     case CIGEMM_ALGO_TILE: ok = launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq); break;
+    case CIGEMM_ALGO_TILE_PAIRED:
+      ok = launch_i8_mfma_paired(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);
+      break;
     case CIGEMM_ALGO_SMALL: ok = false; break;
     case CIGEMM_ALGO_GENERIC: launch_generic_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq); break;
     default:

@@ -21,7 +21,6 @@ struct cigemmContext {
   int last_k_splits;   // K ranges of that launch
   int last_waves;      // wavefronts per workgroup of that launch
   int last_per_cu;     // workgroups of that launch resident per compute unit (1 or 2)
-  int tile2_mode;      // which shapes take the two-workgroups-per-unit tile kernel (see capi.hip)
   int first_tile_rows; // when the call took two launches: rows and waves of the first, else 0
   int first_waves;
   char kernel_name[96];  // storage for names composed per call (last_kernel may point here)
@@ -232,6 +231,14 @@ void launch_f32_small(cigemmContext*, int64_t M, int64_t N, int64_t K, const flo
 bool launch_16b_mfma(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
                      const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                      uint16_t* C, int64_t ldc);
+// The two-workgroups-per-unit form of the tile kernel (mfma_tile2.h), K x N operands only;
+// chosen only by cigemmSetAlgo(CIGEMM_ALGO_TILE_PAIRED).
+bool launch_16b_mfma_paired(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
+                            const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
+                            uint16_t* C, int64_t ldc);
+bool launch_i8_mfma_paired(cigemmContext*, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                           int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
+                           int64_t ldc, const DequantArgs* dq);
 // gemm_i8.hip
 bool launch_i8_mfma(cigemmContext*, int64_t M, int64_t N, int64_t K, const int8_t* A,
                     int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,

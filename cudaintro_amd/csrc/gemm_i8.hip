@@ -53,9 +53,9 @@ bool launch_layout(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const in
 
 }  // namespace
 
-bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
-                    int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C, int64_t ldc,
-                    const DequantArgs* dq) {
+static bool i8_tile_ok(int64_t M, int64_t N, int64_t K, const int8_t* A, int64_t lda,
+                       const int8_t* B, int64_t ldb, bool b_nk, const int32_t* C, int64_t ldc,
+                       const DequantArgs* dq) {
   if (!tile::tile_shape_ok(M, N, K, 1, A, lda, B, ldb, !b_nk)) return false;
   if (!dq) {
     if (ldc % 4 || ((uintptr_t)C & 15)) return false;
@@ -65,12 +65,24 @@ bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const i
     if (dq->sb_vec && ((uintptr_t)dq->sb & 15)) return false;
     if (dq->acc_out && (dq->ldacc % 4 || ((uintptr_t)dq->acc_out & 15))) return false;
   }
-  bool split = false;
-  if (!b_nk && ctx->tile2_mode == 1)
-    launch_kn_tile2(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
-  else
-    split = b_nk ? launch_layout<tile::B_NK>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq)
-                 : launch_layout<tile::B_KN8>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
+  return true;
+}
+
+bool launch_i8_mfma_paired(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                           int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
+                           int64_t ldc, const DequantArgs* dq) {
+  if (b_nk || !i8_tile_ok(M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq)) return false;
+  launch_kn_tile2(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
+  set_tile_kernel_name(ctx, "i8", 64, dq ? "_kn_dequant" : "_kn", false);
+  return true;
+}
+
+bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                    int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C, int64_t ldc,
+                    const DequantArgs* dq) {
+  if (!i8_tile_ok(M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq)) return false;
+  const bool split = b_nk ? launch_layout<tile::B_NK>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq)
+                          : launch_layout<tile::B_KN8>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
   set_tile_kernel_name(ctx, "i8", 64, dq ? (b_nk ? "_nk_dequant" : "_kn_dequant") : (b_nk ? "_nk" : "_kn"),
                        split);
   return true;

@@ -124,7 +124,12 @@ typedef enum cigemmAlgo {
   CIGEMM_ALGO_GENERIC = 0, /* any-shape scalar kernel (fp32: bit-exact with the CPU loop) */
   CIGEMM_ALGO_TILE = 1,    /* LDS-tiled MFMA kernel, 256-column tiles */
   CIGEMM_ALGO_SKINNY = 2,  /* M <= 32 weight-streaming kernels (16-bit K x N, int8 N x K) */
-  CIGEMM_ALGO_SMALL = 3    /* fp32 32x32 tile per workgroup, k split over the waves */
+  CIGEMM_ALGO_SMALL = 3,   /* fp32 32x32 tile per workgroup, k split over the waves */
+  CIGEMM_ALGO_TILE_PAIRED = 4 /* LDS-tiled MFMA kernel with 128-row tiles, two workgroups resident
+                              per compute unit and out of phase (16-bit, int8 K x N).  Never
+                              chosen by DEFAULT: it issues more matrix instructions per cycle and
+                              is slower on a power-limited chip; kept selectable as the measured
+                              counterpart of CIGEMM_ALGO_TILE */
 } cigemmAlgo_t;
 CIGEMM_API cigemmStatus_t cigemmSetAlgo(cigemmHandle_t handle, cigemmAlgo_t algo);
 CIGEMM_API cigemmStatus_t cigemmGetAlgo(cigemmHandle_t handle, cigemmAlgo_t* algo);
@@ -248,7 +253,9 @@ CIGEMM_API cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t handle, int kind, int
  * matrix-core kernel (the product kernel with four timestamps added per workgroup) on the
  * handle's stream, waits for it, and reduces the stamps: kind 0 = bf16 (A, B, C as in
  * cigemm_gemm_bf16), 1 = int8 K x N operands, int32 out (as cigemm_gemm_i8_i32 with
- * CIGEMM_B_KN).  Same shape and alignment conditions as the tile kernel, N % 8 == 0.
+ * CIGEMM_B_KN); 2 and 3 = the same two on the CIGEMM_ALGO_TILE_PAIRED form of the kernel
+ * (128-row tiles; "stage" then means a stage of such a tile, 512 matrix-core issue cycles
+ * instead of 1024).  Same shape and alignment conditions as the tile kernel, N % 8 == 0.
  * phases[0..7] receive, averaged over the workgroups: microseconds from workgroup start to the
  * first stage in registers; of the main loop; of the epilogue until its stores are
  * acknowledged; microseconds from the first workgroup's start to the last one's end; shader

@@ -29,17 +29,19 @@ def test_probe_output_equals_plain_call_and_phases_add_up(handle, torch_gpu, ora
         out = torch.zeros((M, N), dtype=torch.int32, device="cuda")
         with handle.algo(ci.ALGO_TILE):
             want = handle.gemm_i8_i32(a, b, ci.B_KN)
-    ph = handle.probe_tile_phases(a, b, out)
-    assert handle.last_kernel == "tile_phase_probe"
-    assert torch.equal(out.view(torch.uint8), want.view(torch.uint8))
-    tiles = -(-M // 256) * -(-N // 256)
-    assert ph["workgroups"] == tiles
-    assert ph["prologue_us"] > 0 and ph["main_loop_us"] > 0 and ph["epilogue_us"] > 0
-    # one workgroup's phases fit inside the launch; the matrix cores cannot issue a stage of
-    # the 256 x 256 tile in fewer than 1024 cycles; the clock is a plausible one
-    assert ph["prologue_us"] + ph["main_loop_us"] + ph["epilogue_us"] <= ph["first_start_to_last_end_us"] * 1.001
-    assert ph["cycles_per_stage"] >= 1024
-    assert 0.5 < ph["main_loop_clock_ghz"] < 2.6
+    for paired, rows, min_cycles in ((False, 256, 1024), (True, 128, 512)):
+        out.zero_()
+        ph = handle.probe_tile_phases(a, b, out, paired=paired)
+        assert handle.last_kernel == "tile_phase_probe"
+        assert torch.equal(out.view(torch.uint8), want.view(torch.uint8))
+        tiles = -(-M // rows) * -(-N // 256)
+        assert ph["workgroups"] == tiles
+        assert ph["prologue_us"] > 0 and ph["main_loop_us"] > 0 and ph["epilogue_us"] > 0
+        # one workgroup's phases fit inside the launch; the matrix cores cannot issue a stage
+        # of the tile in fewer cycles than its matrix instructions take; the clock is plausible
+        assert ph["prologue_us"] + ph["main_loop_us"] + ph["epilogue_us"] <= ph["first_start_to_last_end_us"] * 1.001
+        assert ph["cycles_per_stage"] >= min_cycles
+        assert 0.5 < ph["main_loop_clock_ghz"] < 2.6
 
 
 def test_probe_rejects_bad_arguments(handle, torch_gpu):
