@@ -236,7 +236,27 @@ def k_sweep(torch, ci, wl, handle, steps, warmup):
         res[name]["fit"] = {"a_us_per_tile": a_us, "b_us_per_stage": b_us}
         log(f"[k-sweep] {name}: {json.dumps(res[name])}")
         del a, b, out
-    print(json.dumps({"k_sweep": res}), flush=True)
+    # Phases of one instrumented launch while 1, 16, 64, 128, 256 and 1024 workgroups are
+    # resident (M = N from 256 to 8192 at K = 4096): the cycles per stage stay, the clock the
+    # chip holds under the load does not.
+    occ = {}
+    r = np.random.Generator(np.random.PCG64(1))
+    for kind in ("int8", "bf16"):
+        for (Mo, No) in ((256, 256), (1024, 1024), (2048, 2048), (2048, 4096), (4096, 4096), (8192, 8192)):
+            if kind == "int8":
+                a = torch.from_numpy(r.integers(-127, 128, size=(Mo, 4096), dtype=np.int8)).cuda()
+                b = torch.from_numpy(r.integers(-127, 128, size=(4096, No), dtype=np.int8)).cuda()
+                o = torch.empty((Mo, No), dtype=torch.int32, device="cuda")
+            else:
+                a = torch.randn((Mo, 4096), device="cuda").to(torch.bfloat16)
+                b = torch.randn((4096, No), device="cuda").to(torch.bfloat16)
+                o = torch.empty((Mo, No), dtype=torch.bfloat16, device="cuda")
+            for _ in range(20):
+                ph = handle.probe_tile_phases(a, b, o)
+            occ[f"{kind}_{Mo}x{No}x4096"] = ph
+            log(f"[occupancy] {kind} {Mo}x{No}x4096: {json.dumps(ph)}")
+            del a, b, o
+    print(json.dumps({"k_sweep": res, "occupancy_sweep": occ}), flush=True)
 
 
 def main():
