@@ -57,17 +57,16 @@ __device__ __forceinline__ void wait_vmcnt_n() {
 // (rem <= MAX_REM; the count of s_waitcnt is an immediate, hence the switch).
 template <int PER_STAGE, int MAX_REM>
 __device__ __forceinline__ void wait_stages_in_flight(int rem) {
-  static_assert(MAX_REM <= 7, "rings of at most 8 stages");
+  static_assert(MAX_REM <= 15 && PER_STAGE * MAX_REM < 64, "vmcnt is a 6-bit counter");
+#define CIG_WAIT_CASE(R) \
+  case R: wait_vmcnt_n<PER_STAGE * (MAX_REM >= R ? R : 0)>(); break;
   switch (rem) {
-    case 0: wait_vmcnt_n<0>(); break;
-    case 1: wait_vmcnt_n<PER_STAGE * (MAX_REM >= 1 ? 1 : 0)>(); break;
-    case 2: wait_vmcnt_n<PER_STAGE * (MAX_REM >= 2 ? 2 : 0)>(); break;
-    case 3: wait_vmcnt_n<PER_STAGE * (MAX_REM >= 3 ? 3 : 0)>(); break;
-    case 4: wait_vmcnt_n<PER_STAGE * (MAX_REM >= 4 ? 4 : 0)>(); break;
-    case 5: wait_vmcnt_n<PER_STAGE * (MAX_REM >= 5 ? 5 : 0)>(); break;
-    case 6: wait_vmcnt_n<PER_STAGE * (MAX_REM >= 6 ? 6 : 0)>(); break;
-    default: wait_vmcnt_n<PER_STAGE * (MAX_REM >= 7 ? 7 : 0)>(); break;
+    CIG_WAIT_CASE(0) CIG_WAIT_CASE(1) CIG_WAIT_CASE(2) CIG_WAIT_CASE(3) CIG_WAIT_CASE(4)
+    CIG_WAIT_CASE(5) CIG_WAIT_CASE(6) CIG_WAIT_CASE(7) CIG_WAIT_CASE(8) CIG_WAIT_CASE(9)
+    CIG_WAIT_CASE(10) CIG_WAIT_CASE(11) CIG_WAIT_CASE(12) CIG_WAIT_CASE(13) CIG_WAIT_CASE(14)
+    default: wait_vmcnt_n<PER_STAGE * MAX_REM>(); break;
   }
+#undef CIG_WAIT_CASE
 }
 
 // ---- 16-bit weights, K x N ------------------------------------------------------------------
@@ -544,6 +543,212 @@ bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, cons
   return false;
 }
 
+// ---- 16-bit, K x N weights, 64-column slabs: K over the waves, at most a two-way exchange ---
+// The kernel above gives a workgroup 256 columns and splits K over up to 16 workgroups per slab,
+// so its reduction reads up to 16 partial tiles per slab.  Here a workgroup owns 64 columns --
+// one whole 128-byte line of every weight row, the narrowest slab whose requests are not half
+// lines -- and a K range; inside it the four waves split k (a stage is 64 rows of k, wave w moves
+// and multiplies rows 16 w .. 16 w + 15 of every stage and never touches what another wave
+// moved: no workgroup barrier in the loop), their four partial 32 x 64 tiles are summed through
+// LDS in wave order, and only then do K ranges meet, through the same partial / arrival-counter
+// exchange as above.  N = 8192 gives 128 slabs, so two K ranges fill 256 compute units: the
+// last workgroup of a slab reads one partial tile instead of seven.
+// Per wave and stage: the W piece [16 k][64 n] (2 KiB, two DMA instructions of 8 whole lines) and
+// the x piece [XR m][16 k] (XR x 32 bytes, one DMA instruction of 2 XR lanes; XR = 8, 16 or 32,
+// the smallest that holds M), in a ring of KW_STAGES slots private to the wave.
+template <int XR_>
+struct KN16KW {
+  static constexpr int BN = 64;
+  static constexpr int K_STAGE = 64;                   // k rows per stage and workgroup
+  static constexpr int XR = XR_;
+  static constexpr int W_BYTES = 16 * 128;             // per wave and stage
+  static constexpr int X_BYTES = XR * 32;
+  static constexpr int SLOT_BYTES = W_BYTES + X_BYTES;
+  static constexpr int NSTAGES = 12;                   // per wave: 27 / 30 / 36 KiB
+  static constexpr int DPS = 3;                        // DMA instructions per wave and stage
+  static constexpr int WAVE_BYTES = NSTAGES * SLOT_BYTES;
+  static constexpr int RED_LD = 68;                    // floats per row of the reduction tiles
+  static constexpr int RED_BYTES = 4 * 32 * RED_LD * 4;
+  static constexpr int LDS_BYTES = 4 * WAVE_BYTES > RED_BYTES ? 4 * WAVE_BYTES : RED_BYTES;
+};
+
+template <typename Math, typename Epi, int XR>
+__global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
+    int M, int N, int stages_per_split, int splits, const char* __restrict__ X, int64_t ldx,
+    const char* __restrict__ W, int64_t ldw, Epi epi, uint64_t* __restrict__ partials,
+    uint32_t* __restrict__ counters) {
+  typedef KN16KW<XR> G;
+  typedef tile::lds_i16x4 lds_i16x4;
+  constexpr int NS = G::NSTAGES, DIST = NS - 1;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  __shared__ int is_last;
+  const int t = threadIdx.x, l = t & 63;
+  const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int slab = blockIdx.x / splits, split = blockIdx.x % splits;
+  const int64_t n0 = (int64_t)slab * G::BN;
+  const int64_t k0 = (int64_t)split * stages_per_split * G::K_STAGE + 16 * w;  // this wave's rows
+  const int KTS = stages_per_split;
+  char* const wave_lds = lds + w * G::WAVE_BYTES;
+  const uint32_t wave_base =
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + w * G::WAVE_BYTES;
+
+  // lane l of a W instruction: row l / 8 of its 8 rows, 16-byte piece l % 8 of the 128-byte line;
+  // of the x instruction (lanes below 2 XR): row l / 2 (rows >= M re-read row M - 1), piece l % 2
+  const char* w_src = W + (k0 + (l >> 3)) * ldw + n0 * 2 + ((l & 7) << 4);
+  const int xm = (l >> 1) < M ? (l >> 1) : M - 1;
+  const char* x_src = X + (int64_t)xm * ldx + k0 * 2 + ((l & 1) << 4);
+  auto issue = [&](int st, int slot) {
+    const uint32_t dst = wave_base + slot * G::SLOT_BYTES;
+    const char* ws = w_src + (int64_t)st * G::K_STAGE * ldw;
+    dma16(ws, dst);
+    dma16(ws + 8 * ldw, dst + 1024);
+    if (l < 2 * XR) dma16(x_src + st * (G::K_STAGE * 2), dst + G::W_BYTES);
+  };
+
+  typename Math::acc_t acc[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[j][e] = 0;
+#pragma unroll
+  for (int st = 0; st < DIST; ++st)
+    if (st < KTS) issue(st, st);
+
+  // fragment addresses within a slot: the transposing read of the W piece (within 16 lanes, lane
+  // i supplies 8 bytes of row i / 4 and receives the k-values of column i; lanes 32-63 take rows
+  // 8-15), and 16 bytes of row l % XR of the x piece
+  const int frag_k = 8 * (l >> 5) + ((l & 15) >> 2);
+  const int frag_n = 16 * ((l >> 4) & 1) + 4 * (l & 3);
+  const int w_off = frag_k * 128 + frag_n * 2;
+  const int x_off = G::W_BYTES + (l & (XR - 1)) * 32 + ((l >> 5) << 4);
+  int slot = 0, dma_slot = DIST;
+  for (int s = 0; s < KTS; ++s) {
+    // Stage s landed for this wave; nothing is fetched past the K range, so fewer stages are
+    // in flight at its end.  The slot refilled now is the one of stage s - 1, whose fragments
+    // this wave's own MFMAs have consumed.
+    wait_stages_in_flight<G::DPS, DIST - 1>(KTS - 1 - s < DIST - 1 ? KTS - 1 - s : DIST - 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (s + DIST < KTS) issue(s + DIST, dma_slot);
+    const char* sl = wave_lds + slot * G::SLOT_BYTES;
+    const u32x4 xf = *reinterpret_cast<const u32x4*>(sl + x_off);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(sl + w_off + 64 * j));
+      const i16x4 hi =
+          __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(sl + w_off + 64 * j + 4 * 128));
+      const u32x4 wf = __builtin_shufflevector(__builtin_bit_cast(u32x2, lo),
+                                               __builtin_bit_cast(u32x2, hi), 0, 1, 2, 3);
+      acc[j] = Math::mfma(wf, xf, acc[j]);
+    }
+    slot = slot + 1 == NS ? 0 : slot + 1;
+    dma_slot = dma_slot + 1 == NS ? 0 : dma_slot + 1;
+  }
+  __syncthreads();  // every wave done with its ring (nothing is in flight): reuse it
+
+  // acc[j][4 q + e] = this wave's part of y[l % 32][n0 + 32 j + 8 q + 4 (l / 32) + e]
+  float* red = reinterpret_cast<float*>(lds);  // [4 waves][32 m][RED_LD]
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x4 v = {acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]};
+      *reinterpret_cast<f32x4*>(red + (w * 32 + (l & 31)) * G::RED_LD + 32 * j + 8 * q +
+                                4 * (l >> 5)) = v;
+    }
+  __syncthreads();
+  // thread t: row t / 8, columns 8 (t % 8) .. + 7, summed over the waves in wave order
+  const int m = t >> 3, c = (t & 7) * 8;
+  float sum[8];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    f32x4 v = *reinterpret_cast<const f32x4*>(red + m * G::RED_LD + c + 4 * h);
+#pragma unroll
+    for (int ww = 1; ww < 4; ++ww) {
+      const f32x4 p = *reinterpret_cast<const f32x4*>(red + (ww * 32 + m) * G::RED_LD + c + 4 * h);
+      v += p;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum[4 * h + e] = v[e];
+  }
+  if (splits == 1) {
+    if (m < M) {
+      epi(m, n0 + c, sum[0], sum[1], sum[2], sum[3]);
+      epi(m, n0 + c + 4, sum[4], sum[5], sum[6], sum[7]);
+    }
+    return;
+  }
+  // ---- K ranges meet: same exchange as in skinny_kernel (partials as agent-scope 64-bit words,
+  // laid out [split][slab][word][thread]; the last workgroup of the slab sums in split order)
+  const int slabs = gridDim.x / splits;
+  auto part = [&](int sp) { return partials + ((int64_t)(sp * slabs + slab) * 4) * 256 + t; };
+  if (m < M) {
+    uint64_t* dst = part(split);
+    store_partial(dst, sum[0], sum[1], sum[2], sum[3]);
+    store_partial(dst + 512, sum[4], sum[5], sum[6], sum[7]);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's partial stores are acknowledged
+  __syncthreads();
+  if (t == 0) {
+    const uint32_t old = __hip_atomic_fetch_add(counters + slab, 1u, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+    is_last = old == (uint32_t)(splits - 1);
+  }
+  __syncthreads();
+  if (!is_last) return;
+  if (m < M) {
+    float lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
+    for (int sp = 0; sp < splits; ++sp) {
+      add_partial(part(sp), lo);
+      add_partial(part(sp) + 512, hi);
+    }
+    epi(m, n0 + c, lo[0], lo[1], lo[2], lo[3]);
+    epi(m, n0 + c + 4, hi[0], hi[1], hi[2], hi[3]);
+  }
+  if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// K ranges for the kernel above: a power of two, enough workgroups to cover the chip about once,
+// at least 8 stages per range, partials and counters within the workspace.
+inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts) {
+  const int64_t slabs = N / 64;
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  int s = 1;
+  while (s < 16 && slabs * s < cus && kts % (2 * s) == 0 && kts / (2 * s) >= 8 &&
+         (size_t)(2 * s) * slabs * 8192 <= ctx->ws_partial_bytes)
+    s *= 2;
+  if ((size_t)slabs * 4 > ctx->ws_counter_bytes) s = 1;
+  return s;
+}
+
+template <typename Math, typename Epi, int XR>
+void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
+                           int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
+  typedef KN16KW<XR> G;
+  static_assert(G::LDS_BYTES <= 160 * 1024, "rings must fit the LDS");
+  auto kern = skinny_kn16_kwaves_kernel<Math, Epi, XR>;
+  static std::atomic<uint64_t> lds_set{0};
+  ensure_dynamic_lds(ctx, (const void*)kern, G::LDS_BYTES, lds_set);
+  const int64_t kts = K / G::K_STAGE;
+  const int splits = kn16_kwaves_splits(ctx, N, kts);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN * splits)), dim3(256), G::LDS_BYTES,
+                     ctx->stream, (int)M, (int)N, (int)(kts / splits), splits,
+                     static_cast<const char*>(X), ldx_bytes, static_cast<const char*>(W),
+                     ldw_bytes, epi, static_cast<uint64_t*>(ctx->workspace),
+                     reinterpret_cast<uint32_t*>(static_cast<char*>(ctx->workspace) +
+                                                 ctx->ws_partial_bytes));
+}
+
+template <typename Math, typename Epi>
+void launch_kn16_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
+                        int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
+  if (M <= 8)
+    launch_kn16_kwaves_xr<Math, Epi, 8>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+  else if (M <= 16)
+    launch_kn16_kwaves_xr<Math, Epi, 16>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+  else
+    launch_kn16_kwaves_xr<Math, Epi, 32>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+}
+
 template <typename Geo>
 bool skinny_shape_ok(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K, int elem,
                      const void* X, int64_t ldx, const void* W, int64_t ldw) {
@@ -561,22 +766,43 @@ struct Slab32 {
   static constexpr int BN = 32, K_ELEMS = 128;
 };
 
+// Which 16-bit decode kernel.  The 64-column one needs whole stages of 64 k per range and pays
+// for its narrow slabs with four times the x traffic of the 256-column one: faster everywhere
+// (N = K = 4096: 19.4 -> 11.9 us, 2048 x 8192: 19.4 -> 13.0, N = K = 8192: 30.9 -> 30.0 at M = 1,
+// 31.2 -> 30.5 at M = 16) except with more than 16 rows of x over many slabs (M = 32 at N = K =
+// 8192: 32.7 against 34.1 us; at N = K = 4096 still 20.3 -> 12.7).
+inline bool kn16_use_kwaves(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K) {
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  if (N % 64 || K % 64 || (size_t)(N / 64) * 4 > ctx->ws_counter_bytes) return false;
+  return M <= 16 || N / 64 < cus / 2;
+}
+
+// Policy + launch of the 16-bit decode GEMM on a context whose workspace is in place (a handle's,
+// or the static array of the entry point that allocates nothing): both must make the same
+// choices so that they give the same bits.  Returns the kernel's name.
+template <typename Math, typename E16>
+const char* launch_skinny_16_on(cigemmContext* ctx, int64_t M, int64_t N, int64_t K,
+                                const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
+                                uint16_t* C, int64_t ldc, bool bf16) {
+  if (kn16_use_kwaves(ctx, M, N, K)) {
+    launch_kn16_kwaves<Math>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
+    return bf16 ? "bf16_skinny_32x64_kwaves" : "f16_skinny_32x64_kwaves";
+  }
+  launch_skinny<GeoKN16<Math>>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
+  return bf16 ? "bf16_skinny_32x256_ring8" : "f16_skinny_32x256_ring8";
+}
+
 }  // namespace
 
 bool launch_skinny_16(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_t K,
                       const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, uint16_t* C,
                       int64_t ldc) {
   typedef GeoKN16<tile::MathBF16> GB;
-  typedef GeoKN16<tile::MathF16> GF;
   if (!skinny_shape_ok<GB>(ctx, M, N, K, 2, A, lda, B, ldb)) return false;
   if (ldc % 4 || ((uintptr_t)C & 7)) return false;
-  if (bf16) {
-    launch_skinny<GB>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<BF16>{C, ldc});
-    ctx->last_kernel = "bf16_skinny_32x256_ring8";
-  } else {
-    launch_skinny<GF>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<F16>{C, ldc});
-    ctx->last_kernel = "f16_skinny_32x256_ring8";
-  }
+  ctx->last_kernel =
+      bf16 ? launch_skinny_16_on<tile::MathBF16, BF16>(ctx, M, N, K, A, lda, B, ldb, C, ldc, true)
+           : launch_skinny_16_on<tile::MathF16, F16>(ctx, M, N, K, A, lda, B, ldb, C, ldc, false);
   return true;
 }
 
@@ -741,12 +967,13 @@ extern "C" cigemmStatus_t cigemm_gemm_bf16_static(void* stream, int64_t M, int64
                        "%s: needs N %% 256 == 0, K %% 32 == 0, lda and ldb multiples of 8, ldc of "
                        "4, A and B 16-byte and C 8-byte aligned (M=%lld N=%lld K=%lld)",
                        name, (long long)M, (long long)N, (long long)K);
-  if (choose_splits<GB>(&ctx, N, K / GB::K_ELEMS) > 1) {
-    const int slabs = (int)(N / GB::BN);
+  {
+    // every arrival counter either kernel may use (one per 64-column slab at most)
+    const int slabs = (int)((N + 63) / 64);
     hipLaunchKernelGGL(clear_counters_kernel, dim3((slabs + 255) / 256), dim3(256), 0, ctx.stream,
                        reinterpret_cast<uint32_t*>(sd->ptr + kStaticPartialBytes), slabs);
   }
-  launch_skinny<GB>(&ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<BF16>{C, ldc});
+  (void)launch_skinny_16_on<tile::MathBF16, BF16>(&ctx, M, N, K, A, lda, B, ldb, C, ldc, true);
   if (ctx.pending_error[0]) {
     (void)hipGetLastError();
     return static_fail(err, err_len, CIGEMM_STATUS_INTERNAL_ERROR, "%s: %s", name,

@@ -180,3 +180,32 @@ def test_skinny_workspace_reuse_with_alternating_inputs(handle, torch_gpu, oracl
         y = handle.gemm_bf16(x, w)
         assert "skinny" in handle.last_kernel, handle.last_kernel
         np.testing.assert_array_equal(bits(torch, y), want, err_msg=f"call {i}")
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("M,N,K,kernel", [
+    (1, 256, 64, "32x64_kwaves"), (3, 512, 1024, "32x64_kwaves"), (8, 8192, 8192, "32x64_kwaves"),
+    (16, 8192, 4096, "32x64_kwaves"), (17, 4096, 4096, "32x64_kwaves"), (32, 2048, 8192, "32x64_kwaves"),
+    (32, 256, 3072, "32x64_kwaves"), (5, 16384, 2048, "32x64_kwaves"),
+    (17, 8192, 1024, "32x256_ring8"), (32, 8192, 8192, "32x256_ring8"),     # many rows of x over many slabs
+    (4, 1024, 4096 + 32, "32x256_ring8"),                                     # K not in whole 64-row stages
+])
+def test_skinny_16bit_both_kernels_exact_inputs(handle, torch_gpu, oracle, rng, kind, M, N, K, kernel):
+    """The two 16-bit decode kernels (64-column slabs with K over the waves; 256-column slabs with
+    K over workgroups): which one the shape gets, and bit-equality with the CPU loop on
+    exact-arithmetic inputs, three calls in a row over guard rows."""
+    torch = torch_gpu
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    narrow = oracle.f32_to_bf16 if kind == "bf16" else oracle.f32_to_f16
+    X, W = rng.choice(vals, size=(M, K)), rng.choice(vals, size=(K, N))
+    W[rng.random(size=W.shape) < 0.5] = 0
+    want = narrow(oracle.gemm_f32(X, W))
+    fn = handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16
+    out = torch.full((M + 2, N), 7.0, dtype=torch.bfloat16 if kind == "bf16" else torch.float16, device="cuda")
+    x, w = to_dev(torch, narrow(X), kind), to_dev(torch, narrow(W), kind)
+    for _ in range(3):
+        fn(x, w, out=out[:M])
+        assert handle.last_kernel == f"{kind}_skinny_{kernel}", handle.last_kernel
+        got = bits(torch, out)
+        np.testing.assert_array_equal(got[:M], want)
+        assert (got[M:] == narrow(np.float32(7.0))).all()
