@@ -49,19 +49,20 @@ void set_tile_kernel_name(cigemmContext* ctx, const char* dtype, int k_elems, co
   ctx->last_kernel = ctx->kernel_name;
 }
 
-void ensure_dynamic_lds(cigemmContext* ctx, const void* kernel, int bytes,
+bool ensure_dynamic_lds(cigemmContext* ctx, const void* kernel, int bytes,
                         std::atomic<uint64_t>& done) {
   const uint64_t bit = 1ull << (ctx->device & 63);
-  if (done.load(std::memory_order_acquire) & bit) return;
+  if (done.load(std::memory_order_acquire) & bit) return true;
   const hipError_t e =
       hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (e != hipSuccess) {
     (void)hipGetLastError();
     snprintf(ctx->pending_error, sizeof(ctx->pending_error),
              "the device refused %d bytes of LDS per workgroup (%s)", bytes, hipGetErrorString(e));
-    return;
+    return false;
   }
   done.fetch_or(bit, std::memory_order_release);
+  return true;
 }
 
 namespace {

@@ -51,8 +51,8 @@ void set_tile_kernel_name(cigemmContext* ctx, const char* dtype, int k_elems, co
                           bool splitk);
 // Raises the dynamic-LDS limit of `kernel` to `bytes` once per device and template instance
 // (`done` = that instance's bit mask of devices already set).  A refusal is recorded on the
-// context and reported by check_launch.
-void ensure_dynamic_lds(cigemmContext* ctx, const void* kernel, int bytes,
+// context and reported by check_launch; it returns false and the caller must not launch.
+bool ensure_dynamic_lds(cigemmContext* ctx, const void* kernel, int bytes,
                         std::atomic<uint64_t>& done);
 
 // ---- vector types ---------------------------------------------------------------------

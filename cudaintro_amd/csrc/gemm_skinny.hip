@@ -354,7 +354,7 @@ void launch_skinny_n(cigemmContext* ctx, int64_t M, int64_t N, int64_t kts, cons
   constexpr int LDS_BYTES = Geo::NSTAGES * Geo::STAGE_BYTES;
   auto kern = skinny_kernel<Geo, Epi, SPLITS>;
   static std::atomic<uint64_t> lds_set{0};
-  ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set);
+  if (!ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set)) return;
   const unsigned grid = (unsigned)((N / Geo::BN) * SPLITS);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS_BYTES, ctx->stream, (int)M, (int)N,
                      (int)(kts / SPLITS), static_cast<const char*>(X), ldx_bytes,
@@ -514,7 +514,7 @@ void launch_skinny_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, c
   static_assert(LDS_BYTES <= 160 * 1024, "ring must fit the LDS");
   auto kern = skinny_nk8_kwaves_kernel<Epi, XR>;
   static std::atomic<uint64_t> lds_set{0};
-  ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set);
+  if (!ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set)) return;
   hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN)), dim3(256), LDS_BYTES, ctx->stream, (int)M,
                      (int)N, (int)K, static_cast<const char*>(X), ldx_bytes,
                      static_cast<const char*>(W), ldw_bytes, epi);
@@ -556,30 +556,35 @@ bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, cons
 // Per wave and stage: the W piece [16 k][64 n] (2 KiB, two DMA instructions of 8 whole lines) and
 // the x piece [XR m][16 k] (XR x 32 bytes, one DMA instruction of 2 XR lanes; XR = 8, 16 or 32,
 // the smallest that holds M), in a ring of KW_STAGES slots private to the wave.
-template <int XR_>
+template <int XR_, int NL_>
 struct KN16KW {
-  static constexpr int BN = 64;
+  static constexpr int NL = NL_;                       // 128-byte lines per weight row: 1 or 2
+  static constexpr int BN = 64 * NL;
   static constexpr int K_STAGE = 64;                   // k rows per stage and workgroup
   static constexpr int XR = XR_;
-  static constexpr int W_BYTES = 16 * 128;             // per wave and stage
+  static constexpr int ROW_BYTES = 128 * NL;
+  static constexpr int W_BYTES = 16 * ROW_BYTES;       // per wave and stage
   static constexpr int X_BYTES = XR * 32;
   static constexpr int SLOT_BYTES = W_BYTES + X_BYTES;
-  static constexpr int NSTAGES = 12;                   // per wave: 27 / 30 / 36 KiB
-  static constexpr int DPS = 3;                        // DMA instructions per wave and stage
+  static constexpr int NSTAGES = NL == 1 ? 12 : 7;     // per wave: 27 / 30 / 36 KiB, 35 KiB
+  static constexpr int DPS = 2 * NL + 1;               // DMA instructions per wave and stage
   static constexpr int WAVE_BYTES = NSTAGES * SLOT_BYTES;
-  static constexpr int RED_LD = 68;                    // floats per row of the reduction tiles
+  static constexpr int RED_LD = BN + 4;                // floats per row of the reduction tiles
   static constexpr int RED_BYTES = 4 * 32 * RED_LD * 4;
   static constexpr int LDS_BYTES = 4 * WAVE_BYTES > RED_BYTES ? 4 * WAVE_BYTES : RED_BYTES;
+  static constexpr int PART_WORDS = 4 * NL;            // 64-bit words per thread of a partial tile
 };
 
-template <typename Math, typename Epi, int XR>
+template <typename Math, typename Epi, int XR, int NL>
 __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
     int M, int N, int stages_per_split, int splits, const char* __restrict__ X, int64_t ldx,
     const char* __restrict__ W, int64_t ldw, Epi epi, uint64_t* __restrict__ partials,
     uint32_t* __restrict__ counters) {
-  typedef KN16KW<XR> G;
+  typedef KN16KW<XR, NL> G;
   typedef tile::lds_i16x4 lds_i16x4;
   constexpr int NS = G::NSTAGES, DIST = NS - 1;
+  constexpr int NT = 2 * NL;                 // 32-column tiles of the slab
+  constexpr int ROWS_PER_DMA = 8 / NL;       // one instruction moves 1 KiB of whole rows
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   __shared__ int is_last;
   const int t = threadIdx.x, l = t & 63;
@@ -592,22 +597,22 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   const uint32_t wave_base =
       (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + w * G::WAVE_BYTES;
 
-  // lane l of a W instruction: row l / 8 of its 8 rows, 16-byte piece l % 8 of the 128-byte line;
+  // lane l of a W instruction: row l / (8 NL) of its rows, 16-byte piece l % (8 NL) of the row;
   // of the x instruction (lanes below 2 XR): row l / 2 (rows >= M re-read row M - 1), piece l % 2
-  const char* w_src = W + (k0 + (l >> 3)) * ldw + n0 * 2 + ((l & 7) << 4);
+  const char* w_src = W + (k0 + l / (8 * NL)) * ldw + n0 * 2 + ((l % (8 * NL)) << 4);
   const int xm = (l >> 1) < M ? (l >> 1) : M - 1;
   const char* x_src = X + (int64_t)xm * ldx + k0 * 2 + ((l & 1) << 4);
   auto issue = [&](int st, int slot) {
     const uint32_t dst = wave_base + slot * G::SLOT_BYTES;
     const char* ws = w_src + (int64_t)st * G::K_STAGE * ldw;
-    dma16(ws, dst);
-    dma16(ws + 8 * ldw, dst + 1024);
+#pragma unroll
+    for (int i = 0; i < 2 * NL; ++i) dma16(ws + (int64_t)(ROWS_PER_DMA * i) * ldw, dst + 1024 * i);
     if (l < 2 * XR) dma16(x_src + st * (G::K_STAGE * 2), dst + G::W_BYTES);
   };
 
-  typename Math::acc_t acc[2];
+  typename Math::acc_t acc[NT];
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[j][e] = 0;
 #pragma unroll
@@ -619,7 +624,7 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   // 8-15), and 16 bytes of row l % XR of the x piece
   const int frag_k = 8 * (l >> 5) + ((l & 15) >> 2);
   const int frag_n = 16 * ((l >> 4) & 1) + 4 * (l & 3);
-  const int w_off = frag_k * 128 + frag_n * 2;
+  const int w_off = frag_k * G::ROW_BYTES + frag_n * 2;
   const int x_off = G::W_BYTES + (l & (XR - 1)) * 32 + ((l >> 5) << 4);
   int slot = 0, dma_slot = DIST;
   for (int s = 0; s < KTS; ++s) {
@@ -632,10 +637,10 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
     const char* sl = wave_lds + slot * G::SLOT_BYTES;
     const u32x4 xf = *reinterpret_cast<const u32x4*>(sl + x_off);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NT; ++j) {
       const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(sl + w_off + 64 * j));
-      const i16x4 hi =
-          __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(sl + w_off + 64 * j + 4 * 128));
+      const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (lds_i16x4*)(sl + w_off + 64 * j + 4 * G::ROW_BYTES));
       const u32x4 wf = __builtin_shufflevector(__builtin_bit_cast(u32x2, lo),
                                                __builtin_bit_cast(u32x2, hi), 0, 1, 2, 3);
       acc[j] = Math::mfma(wf, xf, acc[j]);
@@ -648,7 +653,7 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   // acc[j][4 q + e] = this wave's part of y[l % 32][n0 + 32 j + 8 q + 4 (l / 32) + e]
   float* red = reinterpret_cast<float*>(lds);  // [4 waves][32 m][RED_LD]
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const f32x4 v = {acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]};
@@ -656,11 +661,11 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
                                 4 * (l >> 5)) = v;
     }
   __syncthreads();
-  // thread t: row t / 8, columns 8 (t % 8) .. + 7, summed over the waves in wave order
-  const int m = t >> 3, c = (t & 7) * 8;
-  float sum[8];
+  // thread t: row t / 8, columns 8 NL (t % 8) .. + 8 NL - 1, summed over the waves in wave order
+  const int m = t >> 3, c = (t & 7) * 8 * NL;
+  float sum[8 * NL];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
+  for (int h = 0; h < 2 * NL; ++h) {
     f32x4 v = *reinterpret_cast<const f32x4*>(red + m * G::RED_LD + c + 4 * h);
 #pragma unroll
     for (int ww = 1; ww < 4; ++ww) {
@@ -672,19 +677,23 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   }
   if (splits == 1) {
     if (m < M) {
-      epi(m, n0 + c, sum[0], sum[1], sum[2], sum[3]);
-      epi(m, n0 + c + 4, sum[4], sum[5], sum[6], sum[7]);
+#pragma unroll
+      for (int h = 0; h < 2 * NL; ++h)
+        epi(m, n0 + c + 4 * h, sum[4 * h], sum[4 * h + 1], sum[4 * h + 2], sum[4 * h + 3]);
     }
     return;
   }
   // ---- K ranges meet: same exchange as in skinny_kernel (partials as agent-scope 64-bit words,
   // laid out [split][slab][word][thread]; the last workgroup of the slab sums in split order)
   const int slabs = gridDim.x / splits;
-  auto part = [&](int sp) { return partials + ((int64_t)(sp * slabs + slab) * 4) * 256 + t; };
+  auto part = [&](int sp) {
+    return partials + ((int64_t)(sp * slabs + slab) * G::PART_WORDS) * 256 + t;
+  };
   if (m < M) {
     uint64_t* dst = part(split);
-    store_partial(dst, sum[0], sum[1], sum[2], sum[3]);
-    store_partial(dst + 512, sum[4], sum[5], sum[6], sum[7]);
+#pragma unroll
+    for (int h = 0; h < 2 * NL; ++h)
+      store_partial(dst + 512 * h, sum[4 * h], sum[4 * h + 1], sum[4 * h + 2], sum[4 * h + 3]);
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's partial stores are acknowledged
   __syncthreads();
@@ -696,40 +705,39 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   __syncthreads();
   if (!is_last) return;
   if (m < M) {
-    float lo[4] = {0, 0, 0, 0}, hi[4] = {0, 0, 0, 0};
-    for (int sp = 0; sp < splits; ++sp) {
-      add_partial(part(sp), lo);
-      add_partial(part(sp) + 512, hi);
+#pragma unroll
+    for (int h = 0; h < 2 * NL; ++h) {
+      float q4[4] = {0, 0, 0, 0};
+      for (int sp = 0; sp < splits; ++sp) add_partial(part(sp) + 512 * h, q4);
+      epi(m, n0 + c + 4 * h, q4[0], q4[1], q4[2], q4[3]);
     }
-    epi(m, n0 + c, lo[0], lo[1], lo[2], lo[3]);
-    epi(m, n0 + c + 4, hi[0], hi[1], hi[2], hi[3]);
   }
   if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // K ranges for the kernel above: a power of two, enough workgroups to cover the chip about once,
 // at least 8 stages per range, partials and counters within the workspace.
-inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts) {
-  const int64_t slabs = N / 64;
+inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, int nl) {
+  const int64_t slabs = N / (64 * nl);
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
   int s = 1;
   while (s < 16 && slabs * s < cus && kts % (2 * s) == 0 && kts / (2 * s) >= 8 &&
-         (size_t)(2 * s) * slabs * 8192 <= ctx->ws_partial_bytes)
+         (size_t)(2 * s) * slabs * 8192 * nl <= ctx->ws_partial_bytes)
     s *= 2;
   if ((size_t)slabs * 4 > ctx->ws_counter_bytes) s = 1;
   return s;
 }
 
-template <typename Math, typename Epi, int XR>
+template <typename Math, typename Epi, int XR, int NL>
 void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
                            int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
-  typedef KN16KW<XR> G;
-  static_assert(G::LDS_BYTES <= 160 * 1024, "rings must fit the LDS");
-  auto kern = skinny_kn16_kwaves_kernel<Math, Epi, XR>;
+  typedef KN16KW<XR, NL> G;
+  static_assert(G::LDS_BYTES + 64 <= 160 * 1024, "rings and the arrival flag must fit the LDS");
+  auto kern = skinny_kn16_kwaves_kernel<Math, Epi, XR, NL>;
   static std::atomic<uint64_t> lds_set{0};
-  ensure_dynamic_lds(ctx, (const void*)kern, G::LDS_BYTES, lds_set);
+  if (!ensure_dynamic_lds(ctx, (const void*)kern, G::LDS_BYTES, lds_set)) return;
   const int64_t kts = K / G::K_STAGE;
-  const int splits = kn16_kwaves_splits(ctx, N, kts);
+  const int splits = kn16_kwaves_splits(ctx, N, kts, NL);
   hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN * splits)), dim3(256), G::LDS_BYTES,
                      ctx->stream, (int)M, (int)N, (int)(kts / splits), splits,
                      static_cast<const char*>(X), ldx_bytes, static_cast<const char*>(W),
@@ -738,15 +746,18 @@ void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, 
                                                  ctx->ws_partial_bytes));
 }
 
+// One line per weight row (64-column slabs).  Two lines per row (NL = 2: half the x traffic per
+// weight byte, half as many slabs) was measured for 17 to 32 rows of x: 1 % faster than the
+// 256-column kernel at N = K = 8192, 2-5 % at N = 16384, much slower than NL = 1 below; not used.
 template <typename Math, typename Epi>
 void launch_kn16_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
                         int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
   if (M <= 8)
-    launch_kn16_kwaves_xr<Math, Epi, 8>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    launch_kn16_kwaves_xr<Math, Epi, 8, 1>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
   else if (M <= 16)
-    launch_kn16_kwaves_xr<Math, Epi, 16>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    launch_kn16_kwaves_xr<Math, Epi, 16, 1>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
   else
-    launch_kn16_kwaves_xr<Math, Epi, 32>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    launch_kn16_kwaves_xr<Math, Epi, 32, 1>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
 }
 
 template <typename Geo>

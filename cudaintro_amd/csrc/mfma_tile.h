@@ -862,7 +862,7 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
   constexpr int LDS_BYTES = RING_BYTES > STAGING_BYTES ? RING_BYTES : STAGING_BYTES;
   auto kern = mfma_tile_kernel<Math, BMODE, NSTAGES, MT, Epi, WM>;
   static std::atomic<uint64_t> lds_set{0};  // one per template instance
-  ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set);
+  if (!ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set)) return;
   const int tiles_m = (int)((M + TILE_M - 1) / TILE_M), tiles_n = (int)((N + BN - 1) / BN);
   ctx->last_tile_rows = TILE_M;
   ctx->last_k_splits = splits;

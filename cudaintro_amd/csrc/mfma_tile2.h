@@ -283,7 +283,7 @@ void launch_tile2(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, con
                   int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi) {
   auto kern = mfma_tile2_kernel<Math, BMODE, Epi>;
   static std::atomic<uint64_t> lds_set{0};
-  ensure_dynamic_lds(ctx, (const void*)kern, T2_LDS_BYTES, lds_set);
+  if (!ensure_dynamic_lds(ctx, (const void*)kern, T2_LDS_BYTES, lds_set)) return;
   const int tiles_m = (int)((M + T2_TILE_M - 1) / T2_TILE_M), tiles_n = (int)((N + BN - 1) / BN);
   const int64_t kts = (K_bytes + KB - 1) / KB;
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
