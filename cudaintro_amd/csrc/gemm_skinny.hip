@@ -207,14 +207,42 @@ __device__ __forceinline__ void store_partial(uint64_t* dst, T v0, T v1, T v2, T
   __hip_atomic_store(dst, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __hip_atomic_store(dst + 256, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-template <typename T>
-__device__ __forceinline__ void add_partial(const uint64_t* src, T (&sum)[4]) {
-  const uint64_t lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const uint64_t hi = __hip_atomic_load(src + 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  sum[0] += __builtin_bit_cast(T, (uint32_t)lo);
-  sum[1] += __builtin_bit_cast(T, (uint32_t)(lo >> 32));
-  sum[2] += __builtin_bit_cast(T, (uint32_t)hi);
-  sum[3] += __builtin_bit_cast(T, (uint32_t)(hi >> 32));
+// The reduction of the last workgroup of a slab: NQ quads of this thread, summed over the S
+// partial tiles in split order, each sum starting from zero (the result does not depend on which
+// workgroup arrived last).  `first` = word of (split 0, this slab, quad 0, half 0, this lane),
+// `split_stride` = words between the tiles of consecutive splits.  The loads of up to 32 quads
+// are issued back to back before the first sum waits: a load from the coherence point takes
+// most of a microsecond, and one round trip per quad and split was a third of the time of a
+// 16 MB weight matrix.
+template <typename T, int NQ, int S>
+__device__ __forceinline__ void sum_partials(const uint64_t* first, int64_t split_stride,
+                                             T (&sum)[NQ][4]) {
+  constexpr int CH = S * NQ <= 32 ? S : (32 / NQ > 0 ? 32 / NQ : 1);  // splits per batch
+#pragma unroll
+  for (int q = 0; q < NQ; ++q)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum[q][e] = 0;
+#pragma unroll
+  for (int s0 = 0; s0 < S; s0 += CH) {
+    uint64_t lo[CH][NQ], hi[CH][NQ];
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const uint64_t* src = first + (s0 + c) * split_stride + q * 512;
+        lo[c][q] = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        hi[c][q] = __hip_atomic_load(src + 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        sum[q][0] += __builtin_bit_cast(T, (uint32_t)lo[c][q]);
+        sum[q][1] += __builtin_bit_cast(T, (uint32_t)(lo[c][q] >> 32));
+        sum[q][2] += __builtin_bit_cast(T, (uint32_t)hi[c][q]);
+        sum[q][3] += __builtin_bit_cast(T, (uint32_t)(hi[c][q] >> 32));
+      }
+  }
 }
 
 // Workspace: the partials (see store_partial) followed by one arrival counter per slab.
@@ -322,15 +350,14 @@ __global__ __launch_bounds__(256, 1) void skinny_kernel(int M, int N, int stages
   __syncthreads();
   if (!is_last) return;
   if (m < M) {
+    scalar_t sum[QUADS][4];
+    sum_partials<scalar_t, QUADS, splits>(part(0), (int64_t)slabs * QUADS * 512, sum);
 #pragma unroll
     for (int j = 0; j < Geo::NT; ++j)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        scalar_t sum[4] = {0, 0, 0, 0};
-#pragma unroll
-        for (int sp = 0; sp < splits; ++sp) add_partial(part(sp) + (j * 4 + q) * 512, sum);
-        epi(m, n0 + Geo::col(w, j, q, l), sum[0], sum[1], sum[2], sum[3]);
-      }
+      for (int q = 0; q < 4; ++q)
+        epi(m, n0 + Geo::col(w, j, q, l), sum[4 * j + q][0], sum[4 * j + q][1], sum[4 * j + q][2],
+            sum[4 * j + q][3]);
   }
   if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -554,37 +581,40 @@ bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, cons
 // exchange as above.  N = 8192 gives 128 slabs, so two K ranges fill 256 compute units: the
 // last workgroup of a slab reads one partial tile instead of seven.
 // Per wave and stage: the W piece [16 k][64 n] (2 KiB, two DMA instructions of 8 whole lines) and
-// the x piece [XR m][16 k] (XR x 32 bytes, one DMA instruction of 2 XR lanes; XR = 8, 16 or 32,
-// the smallest that holds M), in a ring of KW_STAGES slots private to the wave.
-template <int XR_, int NL_>
+// the x piece [XR m][16 k] (XR x 32 bytes of the slot, XR = 8, 16 or 32, the smallest that holds
+// M; one DMA instruction of 2 M lanes fills its first M rows), in a ring of NSTAGES slots private
+// to the wave.
+template <int XR_, int COLS_>
 struct KN16KW {
-  static constexpr int NL = NL_;                       // 128-byte lines per weight row: 1 or 2
-  static constexpr int BN = 64 * NL;
+  static constexpr int BN = COLS_;                     // 32 (half a line per weight row), 64, 128
   static constexpr int K_STAGE = 64;                   // k rows per stage and workgroup
   static constexpr int XR = XR_;
-  static constexpr int ROW_BYTES = 128 * NL;
+  static constexpr int ROW_BYTES = 2 * BN;
   static constexpr int W_BYTES = 16 * ROW_BYTES;       // per wave and stage
+  static constexpr int W_DMAS = W_BYTES / 1024;        // one instruction moves 1 KiB of whole rows
   static constexpr int X_BYTES = XR * 32;
   static constexpr int SLOT_BYTES = W_BYTES + X_BYTES;
-  static constexpr int NSTAGES = NL == 1 ? 12 : 7;     // per wave: 27 / 30 / 36 KiB, 35 KiB
-  static constexpr int DPS = 2 * NL + 1;               // DMA instructions per wave and stage
+  static constexpr int NSTAGES = BN == 32 ? 16 : BN == 64 ? 12 : 7;
+  static constexpr int DPS = W_DMAS + 1;               // DMA instructions per wave and stage
   static constexpr int WAVE_BYTES = NSTAGES * SLOT_BYTES;
   static constexpr int RED_LD = BN + 4;                // floats per row of the reduction tiles
   static constexpr int RED_BYTES = 4 * 32 * RED_LD * 4;
   static constexpr int LDS_BYTES = 4 * WAVE_BYTES > RED_BYTES ? 4 * WAVE_BYTES : RED_BYTES;
-  static constexpr int PART_WORDS = 4 * NL;            // 64-bit words per thread of a partial tile
+  static constexpr int PART_WORDS = BN / 16;           // 64-bit words per thread of a partial tile
 };
 
-template <typename Math, typename Epi, int XR, int NL>
+template <typename Math, typename Epi, int XR, int COLS>
 __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
     int M, int N, int stages_per_split, int splits, const char* __restrict__ X, int64_t ldx,
     const char* __restrict__ W, int64_t ldw, Epi epi, uint64_t* __restrict__ partials,
     uint32_t* __restrict__ counters) {
-  typedef KN16KW<XR, NL> G;
+  typedef KN16KW<XR, COLS> G;
   typedef tile::lds_i16x4 lds_i16x4;
   constexpr int NS = G::NSTAGES, DIST = NS - 1;
-  constexpr int NT = 2 * NL;                 // 32-column tiles of the slab
-  constexpr int ROWS_PER_DMA = 8 / NL;       // one instruction moves 1 KiB of whole rows
+  constexpr int NT = COLS / 32;                       // 32-column tiles of the slab
+  constexpr int PIECES = G::ROW_BYTES / 16;           // 16-byte pieces of a slab row
+  constexpr int ROWS_PER_DMA = 64 / PIECES;
+  constexpr int QUADS = COLS / 32;                    // float4 groups per thread of the reduction
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   __shared__ int is_last;
   const int t = threadIdx.x, l = t & 63;
@@ -597,17 +627,18 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   const uint32_t wave_base =
       (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + w * G::WAVE_BYTES;
 
-  // lane l of a W instruction: row l / (8 NL) of its rows, 16-byte piece l % (8 NL) of the row;
-  // of the x instruction (lanes below 2 XR): row l / 2 (rows >= M re-read row M - 1), piece l % 2
-  const char* w_src = W + (k0 + l / (8 * NL)) * ldw + n0 * 2 + ((l % (8 * NL)) << 4);
-  const int xm = (l >> 1) < M ? (l >> 1) : M - 1;
-  const char* x_src = X + (int64_t)xm * ldx + k0 * 2 + ((l & 1) << 4);
+  // lane l of a W instruction: row l / PIECES of its rows, 16-byte piece l % PIECES of the row;
+  // of the x instruction: row l / 2, piece l % 2, lanes of rows below M only (the rows of the
+  // slot past M keep whatever the LDS held: an output row depends on its own row of x alone, and
+  // rows >= M are never stored)
+  const char* w_src = W + (k0 + l / PIECES) * ldw + n0 * 2 + ((l % PIECES) << 4);
+  const char* x_src = X + (int64_t)(l >> 1) * ldx + k0 * 2 + ((l & 1) << 4);
   auto issue = [&](int st, int slot) {
     const uint32_t dst = wave_base + slot * G::SLOT_BYTES;
     const char* ws = w_src + (int64_t)st * G::K_STAGE * ldw;
 #pragma unroll
-    for (int i = 0; i < 2 * NL; ++i) dma16(ws + (int64_t)(ROWS_PER_DMA * i) * ldw, dst + 1024 * i);
-    if (l < 2 * XR) dma16(x_src + st * (G::K_STAGE * 2), dst + G::W_BYTES);
+    for (int i = 0; i < G::W_DMAS; ++i) dma16(ws + (int64_t)(ROWS_PER_DMA * i) * ldw, dst + 1024 * i);
+    if (l < 2 * M) dma16(x_src + st * (G::K_STAGE * 2), dst + G::W_BYTES);
   };
 
   typename Math::acc_t acc[NT];
@@ -661,11 +692,12 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
                                 4 * (l >> 5)) = v;
     }
   __syncthreads();
-  // thread t: row t / 8, columns 8 NL (t % 8) .. + 8 NL - 1, summed over the waves in wave order
-  const int m = t >> 3, c = (t & 7) * 8 * NL;
-  float sum[8 * NL];
+  // thread t: row t / 8, columns 4 QUADS (t % 8) .. + 4 QUADS - 1, summed over the waves in
+  // wave order
+  const int m = t >> 3, c = (t & 7) * 4 * QUADS;
+  float sum[4 * QUADS];
 #pragma unroll
-  for (int h = 0; h < 2 * NL; ++h) {
+  for (int h = 0; h < QUADS; ++h) {
     f32x4 v = *reinterpret_cast<const f32x4*>(red + m * G::RED_LD + c + 4 * h);
 #pragma unroll
     for (int ww = 1; ww < 4; ++ww) {
@@ -678,7 +710,7 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   if (splits == 1) {
     if (m < M) {
 #pragma unroll
-      for (int h = 0; h < 2 * NL; ++h)
+      for (int h = 0; h < QUADS; ++h)
         epi(m, n0 + c + 4 * h, sum[4 * h], sum[4 * h + 1], sum[4 * h + 2], sum[4 * h + 3]);
     }
     return;
@@ -692,7 +724,7 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   if (m < M) {
     uint64_t* dst = part(split);
 #pragma unroll
-    for (int h = 0; h < 2 * NL; ++h)
+    for (int h = 0; h < QUADS; ++h)
       store_partial(dst + 512 * h, sum[4 * h], sum[4 * h + 1], sum[4 * h + 2], sum[4 * h + 3]);
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's partial stores are acknowledged
@@ -705,39 +737,43 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   __syncthreads();
   if (!is_last) return;
   if (m < M) {
-#pragma unroll
-    for (int h = 0; h < 2 * NL; ++h) {
-      float q4[4] = {0, 0, 0, 0};
-      for (int sp = 0; sp < splits; ++sp) add_partial(part(sp) + 512 * h, q4);
-      epi(m, n0 + c + 4 * h, q4[0], q4[1], q4[2], q4[3]);
+    float q4[QUADS][4];
+    const int64_t stride = (int64_t)slabs * G::PART_WORDS * 256;
+    switch (splits) {
+      case 2: sum_partials<float, QUADS, 2>(part(0), stride, q4); break;
+      case 4: sum_partials<float, QUADS, 4>(part(0), stride, q4); break;
+      case 8: sum_partials<float, QUADS, 8>(part(0), stride, q4); break;
+      default: sum_partials<float, QUADS, 16>(part(0), stride, q4); break;
     }
+#pragma unroll
+    for (int h = 0; h < QUADS; ++h) epi(m, n0 + c + 4 * h, q4[h][0], q4[h][1], q4[h][2], q4[h][3]);
   }
   if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // K ranges for the kernel above: a power of two, enough workgroups to cover the chip about once,
 // at least 8 stages per range, partials and counters within the workspace.
-inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, int nl) {
-  const int64_t slabs = N / (64 * nl);
+inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, int cols) {
+  const int64_t slabs = N / cols;
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
   int s = 1;
   while (s < 16 && slabs * s < cus && kts % (2 * s) == 0 && kts / (2 * s) >= 8 &&
-         (size_t)(2 * s) * slabs * 8192 * nl <= ctx->ws_partial_bytes)
+         (size_t)(2 * s) * slabs * 128 * cols <= ctx->ws_partial_bytes)
     s *= 2;
   if ((size_t)slabs * 4 > ctx->ws_counter_bytes) s = 1;
   return s;
 }
 
-template <typename Math, typename Epi, int XR, int NL>
+template <typename Math, typename Epi, int XR, int COLS>
 void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
                            int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
-  typedef KN16KW<XR, NL> G;
+  typedef KN16KW<XR, COLS> G;
   static_assert(G::LDS_BYTES + 64 <= 160 * 1024, "rings and the arrival flag must fit the LDS");
-  auto kern = skinny_kn16_kwaves_kernel<Math, Epi, XR, NL>;
+  auto kern = skinny_kn16_kwaves_kernel<Math, Epi, XR, COLS>;
   static std::atomic<uint64_t> lds_set{0};
   if (!ensure_dynamic_lds(ctx, (const void*)kern, G::LDS_BYTES, lds_set)) return;
   const int64_t kts = K / G::K_STAGE;
-  const int splits = kn16_kwaves_splits(ctx, N, kts, NL);
+  const int splits = kn16_kwaves_splits(ctx, N, kts, COLS);
   hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN * splits)), dim3(256), G::LDS_BYTES,
                      ctx->stream, (int)M, (int)N, (int)(kts / splits), splits,
                      static_cast<const char*>(X), ldx_bytes, static_cast<const char*>(W),
@@ -746,18 +782,21 @@ void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, 
                                                  ctx->ws_partial_bytes));
 }
 
-// One line per weight row (64-column slabs).  Two lines per row (NL = 2: half the x traffic per
-// weight byte, half as many slabs) was measured for 17 to 32 rows of x: 1 % faster than the
-// 256-column kernel at N = K = 8192, 2-5 % at N = 16384, much slower than NL = 1 below; not used.
-template <typename Math, typename Epi>
+// COLS = 64, one line per weight row, is the only width in use.  Two lines per row (128-column
+// slabs: half the x traffic per weight byte, half as many slabs) was measured for 17 to 32 rows
+// of x: 1 % faster than the 256-column kernel at N = K = 8192, 2-5 % at N = 16384, much slower
+// than 64 columns below.  Half a line per row (32-column slabs: 256 slabs at N = 8192, no
+// exchange between workgroups at all) streams at two thirds of the rate: 45 against 30 us at
+// N = K = 8192, 47 against 28 at 16384 x 4096, level only at N = 1024.
+template <typename Math, int COLS, typename Epi>
 void launch_kn16_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
                         int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
   if (M <= 8)
-    launch_kn16_kwaves_xr<Math, Epi, 8, 1>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    launch_kn16_kwaves_xr<Math, Epi, 8, COLS>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
   else if (M <= 16)
-    launch_kn16_kwaves_xr<Math, Epi, 16, 1>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    launch_kn16_kwaves_xr<Math, Epi, 16, COLS>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
   else
-    launch_kn16_kwaves_xr<Math, Epi, 32, 1>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    launch_kn16_kwaves_xr<Math, Epi, 32, COLS>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
 }
 
 template <typename Geo>
@@ -796,7 +835,7 @@ const char* launch_skinny_16_on(cigemmContext* ctx, int64_t M, int64_t N, int64_
                                 const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                                 uint16_t* C, int64_t ldc, bool bf16) {
   if (kn16_use_kwaves(ctx, M, N, K)) {
-    launch_kn16_kwaves<Math>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
+    launch_kn16_kwaves<Math, 64>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
     return bf16 ? "bf16_skinny_32x64_kwaves" : "f16_skinny_32x64_kwaves";
   }
   launch_skinny<GeoKN16<Math>>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});

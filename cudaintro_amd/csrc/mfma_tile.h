@@ -893,6 +893,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
     const uint32_t* p = part + r * N + c;
     // (element-wise: a bit cast applied directly to a vector element misreads it)
     auto as_scalar = [](uint32_t bits) { return __builtin_bit_cast(Scalar, bits); };
+    // (up to seven splits are read before the first add waits for one: the loop is otherwise
+    // one memory round trip per split)
     u32x4 v = *reinterpret_cast<const u32x4*>(p);
     Scalar sum[4];
 #pragma unroll
@@ -900,13 +902,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
       const uint32_t b = v[e];
       sum[e] = as_scalar(b);
     }
-    for (int sp = 1; sp < splits; ++sp) {
-      v = *reinterpret_cast<const u32x4*>(p + sp * split_stride);
+    for (int sp = 1; sp < splits; sp += 7) {
+      u32x4 u[7];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t b = v[e];
-        sum[e] += as_scalar(b);
-      }
+      for (int i = 0; i < 7; ++i)
+        if (sp + i < splits) u[i] = *reinterpret_cast<const u32x4*>(p + (sp + i) * split_stride);
+#pragma unroll
+      for (int i = 0; i < 7; ++i)
+        if (sp + i < splits) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const uint32_t b = u[i][e];
+            sum[e] += as_scalar(b);
+          }
+        }
     }
     epi(r, c, sum[0], sum[1], sum[2], sum[3]);
   }
