@@ -818,48 +818,61 @@ struct Slab32 {
 
 // Which 16-bit decode kernel.  The 64-column one needs whole stages of 64 k per range and pays
 // for its narrow slabs with four times the x traffic of the 256-column one: faster everywhere
-// (N = K = 4096: 19.4 -> 11.9 us, 2048 x 8192: 19.4 -> 13.0, N = K = 8192: 30.9 -> 30.0 at M = 1,
+// (N = K = 4096: 19.4 -> 11.2 us, 2048 x 8192: 19.4 -> 11.5, N = K = 8192: 30.9 -> 30.0 at M = 1,
 // 31.2 -> 30.5 at M = 16) except with more than 16 rows of x over many slabs (M = 32 at N = K =
 // 8192: 32.7 against 34.1 us; at N = K = 4096 still 20.3 -> 12.7).
-inline bool kn16_use_kwaves(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K) {
+// A shape that only one of the two takes (N a multiple of 64 but not of 256; K a multiple of 32
+// but not of 64) goes to that one.  0: neither, 1: 64-column slabs, 2: 256-column slabs.
+inline int kn16_choice(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K) {
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-  if (N % 64 || K % 64 || (size_t)(N / 64) * 4 > ctx->ws_counter_bytes) return false;
-  return M <= 16 || N / 64 < cus / 2;
+  const bool kw_ok = N % 64 == 0 && K % 64 == 0 && (size_t)(N / 64) * 4 <= ctx->ws_counter_bytes;
+  const bool sk_ok = N % GeoKN16<tile::MathBF16>::BN == 0 && K % GeoKN16<tile::MathBF16>::K_ELEMS == 0;
+  if (kw_ok && (M <= 16 || N / 64 < cus / 2 || !sk_ok)) return 1;
+  return sk_ok ? 2 : 0;
 }
 
 // Policy + launch of the 16-bit decode GEMM on a context whose workspace is in place (a handle's,
 // or the static array of the entry point that allocates nothing): both must make the same
-// choices so that they give the same bits.  Returns the kernel's name.
+// choices so that they give the same bits.  Returns the kernel's name, null when neither kernel
+// takes the shape (nothing was launched).
 template <typename Math, typename E16>
 const char* launch_skinny_16_on(cigemmContext* ctx, int64_t M, int64_t N, int64_t K,
                                 const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                                 uint16_t* C, int64_t ldc, bool bf16) {
-  if (kn16_use_kwaves(ctx, M, N, K)) {
+  const int which = kn16_choice(ctx, M, N, K);
+  if (which == 1) {
     launch_kn16_kwaves<Math, 64>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
     return bf16 ? "bf16_skinny_32x64_kwaves" : "f16_skinny_32x64_kwaves";
   }
+  if (which == 0) return nullptr;
   launch_skinny<GeoKN16<Math>>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
   return bf16 ? "bf16_skinny_32x256_ring8" : "f16_skinny_32x256_ring8";
 }
 
 }  // namespace
 
+// the alignment conditions common to both 16-bit kernels; kn16_choice has the shape conditions
+struct Slab16Any {
+  static constexpr int BN = 64, K_ELEMS = 32;
+};
+
 bool launch_skinny_16(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_t K,
                       const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, uint16_t* C,
                       int64_t ldc) {
-  typedef GeoKN16<tile::MathBF16> GB;
-  if (!skinny_shape_ok<GB>(ctx, M, N, K, 2, A, lda, B, ldb)) return false;
+  if (!skinny_shape_ok<Slab16Any>(ctx, M, N, K, 2, A, lda, B, ldb)) return false;
   if (ldc % 4 || ((uintptr_t)C & 7)) return false;
-  ctx->last_kernel =
+  const char* name =
       bf16 ? launch_skinny_16_on<tile::MathBF16, BF16>(ctx, M, N, K, A, lda, B, ldb, C, ldc, true)
            : launch_skinny_16_on<tile::MathF16, F16>(ctx, M, N, K, A, lda, B, ldb, C, ldc, false);
+  if (!name) return false;
+  ctx->last_kernel = name;
   return true;
 }
 
 bool launch_skinny_i8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
                       int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
                       int64_t ldc, const DequantArgs* dq) {
-  if (!b_nk) return false;  // K x N int8 weights at M <= 32 go to the any-shape kernel
+  if (!b_nk) return false;  // K x N int8 weights at M <= 32 go to the tile kernel (64-row tiles)
   if (!skinny_shape_ok<Slab32>(ctx, M, N, K, 1, A, lda, B, ldb)) return false;
   if (!dq) {
     if (ldc % 4 || ((uintptr_t)C & 15)) return false;

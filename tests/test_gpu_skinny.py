@@ -189,6 +189,8 @@ def test_skinny_workspace_reuse_with_alternating_inputs(handle, torch_gpu, oracl
     (32, 256, 3072, "32x64_kwaves"), (5, 16384, 2048, "32x64_kwaves"),
     (17, 8192, 1024, "32x256_ring8"), (32, 8192, 8192, "32x256_ring8"),     # many rows of x over many slabs
     (4, 1024, 4096 + 32, "32x256_ring8"),                                     # K not in whole 64-row stages
+    (3, 320, 192, "32x64_kwaves"), (20, 8192 + 64, 128, "32x64_kwaves"),     # N in whole lines, not in 256s
+    (32, 16384 + 192, 64, "32x64_kwaves"),
 ])
 def test_skinny_16bit_both_kernels_exact_inputs(handle, torch_gpu, oracle, rng, kind, M, N, K, kernel):
     """The two 16-bit decode kernels (64-column slabs with K over the waves; 256-column slabs with
