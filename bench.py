@@ -415,6 +415,22 @@ def main():
                                                    "ms_over_aligned": e / steps_x / (ev / args.steps),
                                                    "kernel": handle.last_kernel}
             del a, b, c
+        # shapes no aligned kernel takes (odd N: rows of B and C at every 2-byte alignment; odd K:
+        # rows of A): the any-shape matrix-core kernel, and the scalar kernel it took them from
+        for (Mx, Nx, Kx) in ((4096, 4095, 4096), (4096, 4096, 4095)):
+            a_b, b_b = wl.normal_16bit(Mx, Nx, Kx, seed=2, kind="bf16")
+            a, b = dev16(torch, a_b, "bf16"), dev16(torch, b_b, "bf16")
+            c = torch.empty((Mx, Nx), dtype=torch.bfloat16, device="cuda")
+            w, e = time_calls(torch, lambda: handle.gemm_bf16(a, b, out=c), 20, 5)
+            t = wl.gemm_ops(Mx, Nx, Kx) * 20 / e / 1e12
+            name_a = handle.last_kernel
+            with handle.algo(ci.ALGO_GENERIC):
+                w, e_s = time_calls(torch, lambda: handle.gemm_bf16(a, b, out=c), 3, 1)
+            per_config[f"bf16_{Mx}x{Nx}x{Kx}_unaligned"] = {
+                "tflops": t, "frac_of_peak": t / PEAK_16BIT_TFLOPS, "peak": PEAK_16BIT_TFLOPS,
+                "ms": e / 20 * 1e3, "kernel": name_a,
+                "scalar_kernel_tflops": wl.gemm_ops(Mx, Nx, Kx) * 3 / e_s / 1e12}
+            del a, b, c
         per_config[f"bf16_{n}"] = {"tflops": achieved, "frac_of_peak": achieved / PEAK_16BIT_TFLOPS,
                                    "peak": PEAK_16BIT_TFLOPS, "ms": ev / args.steps * 1e3,
                                    "kernel": kernel}

@@ -15,6 +15,7 @@ from .cigemm import (  # noqa: F401
     ALGO_SMALL,
     ALGO_TILE,
     ALGO_TILE_PAIRED,
+    ALGO_MFMA_ANY,
     B_KN,
     B_NK,
     OUT_BF16,

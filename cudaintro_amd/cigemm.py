@@ -17,7 +17,7 @@ _SUITE = os.path.join(_HERE, "gemm_suite")
 
 B_KN, B_NK = 0, 1
 ACT_NONE, ACT_RELU = 0, 1
-ALGO_DEFAULT, ALGO_GENERIC, ALGO_TILE, ALGO_SKINNY, ALGO_SMALL, ALGO_TILE_PAIRED = -1, 0, 1, 2, 3, 4
+ALGO_DEFAULT, ALGO_GENERIC, ALGO_TILE, ALGO_SKINNY, ALGO_SMALL, ALGO_TILE_PAIRED, ALGO_MFMA_ANY = -1, 0, 1, 2, 3, 4, 5
 SCALE_TENSOR, SCALE_VECTOR = 0, 1
 OUT_F32, OUT_BF16 = 0, 1
 

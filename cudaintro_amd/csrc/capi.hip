@@ -209,7 +209,7 @@ cigemmStatus_t cigemmGetLastPlan(cigemmHandle_t h, int* tile_rows, int* k_splits
 
 cigemmStatus_t cigemmSetAlgo(cigemmHandle_t h, cigemmAlgo_t algo) {
   if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
-  if ((int)algo < CIGEMM_ALGO_DEFAULT || (int)algo > CIGEMM_ALGO_TILE_PAIRED)
+  if ((int)algo < CIGEMM_ALGO_DEFAULT || (int)algo > CIGEMM_ALGO_MFMA_ANY)
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "cigemmSetAlgo: bad algo %d", (int)algo);
   h->algo = (int)algo;
   return CIGEMM_STATUS_SUCCESS;
@@ -241,6 +241,7 @@ static bool dispatch_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K, cons
       return true;
     case CIGEMM_ALGO_SKINNY:
     case CIGEMM_ALGO_TILE_PAIRED:
+    case CIGEMM_ALGO_MFMA_ANY:
       return false;
     case CIGEMM_ALGO_GENERIC:
       launch_generic_f32(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
@@ -290,11 +291,14 @@ static cigemmStatus_t gemm16(cigemmHandle_t h, const char* name, bool bf16, int6
       ok = launch_16b_mfma_paired(h, bf16, M, N, K, A, lda, B, ldb, C, ldc);
       break;
     case CIGEMM_ALGO_SMALL: ok = false; break;
+    case CIGEMM_ALGO_MFMA_ANY: ok = launch_mfma_any_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
     case CIGEMM_ALGO_GENERIC: launch_generic_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
     default:
-      // decode shapes (M <= 32) first: they are bandwidth problems with their own kernel
+      // decode shapes (M <= 32) first: they are bandwidth problems with their own kernel; what
+      // neither that nor the tile kernel takes (odd N, unaligned rows) stays on the matrix cores
       if (!launch_skinny_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc) &&
-          !launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc))
+          !launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc) &&
+          !launch_mfma_any_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc))
         launch_generic_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc);
   }
   if (!ok) return algo_refused(h, name);
@@ -326,10 +330,14 @@ static cigemmStatus_t gemm_i8(cigemmHandle_t h, const char* name, int64_t M, int
       ok = launch_i8_mfma_paired(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);
       break;
     case CIGEMM_ALGO_SMALL: ok = false; break;
+    case CIGEMM_ALGO_MFMA_ANY:
+      ok = launch_mfma_any_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);
+      break;
     case CIGEMM_ALGO_GENERIC: launch_generic_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq); break;
     default:
       if (!launch_skinny_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq) &&
-          !launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq))
+          !launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq) &&
+          !launch_mfma_any_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq))
         launch_generic_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);
   }
   if (!ok) return algo_refused(h, name);

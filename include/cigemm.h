@@ -125,11 +125,14 @@ typedef enum cigemmAlgo {
   CIGEMM_ALGO_TILE = 1,    /* LDS-tiled MFMA kernel, 256-column tiles */
   CIGEMM_ALGO_SKINNY = 2,  /* M <= 32 weight-streaming kernels (16-bit K x N, int8 N x K) */
   CIGEMM_ALGO_SMALL = 3,   /* fp32 32x32 tile per workgroup, k split over the waves */
-  CIGEMM_ALGO_TILE_PAIRED = 4 /* LDS-tiled MFMA kernel with 128-row tiles, two workgroups resident
+  CIGEMM_ALGO_TILE_PAIRED = 4, /* LDS-tiled MFMA kernel with 128-row tiles, two workgroups resident
                               per compute unit and out of phase (16-bit, int8 K x N).  Never
                               chosen by DEFAULT: it issues more matrix instructions per cycle and
                               is slower on a power-limited chip; kept selectable as the measured
                               counterpart of CIGEMM_ALGO_TILE */
+  CIGEMM_ALGO_MFMA_ANY = 5 /* 16-bit and int8: 128x128 MFMA tiles fed by element-wise, bounds-checked
+                              loads and stores: any shape, leading dimension and alignment.
+                              DEFAULT uses it for what the families above do not take */
 } cigemmAlgo_t;
 CIGEMM_API cigemmStatus_t cigemmSetAlgo(cigemmHandle_t handle, cigemmAlgo_t algo);
 CIGEMM_API cigemmStatus_t cigemmGetAlgo(cigemmHandle_t handle, cigemmAlgo_t* algo);

@@ -68,7 +68,7 @@ def test_kernel_family_selection(torch_gpu):
     torch = torch_gpu
     h = ci.Handle()
     assert h.get_algo() == ci.ALGO_DEFAULT
-    assert h.lib.cigemmSetAlgo(h.raw, 5) == Status.INVALID_VALUE
+    assert h.lib.cigemmSetAlgo(h.raw, 6) == Status.INVALID_VALUE
     assert h.lib.cigemmSetAlgo(h.raw, -2) == Status.INVALID_VALUE
     assert h.lib.cigemmGetAlgo(h.raw, None) == Status.INVALID_VALUE
     a = torch.ones((64, 64), dtype=torch.float32, device="cuda")

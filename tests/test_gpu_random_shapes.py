@@ -10,7 +10,7 @@ from gpu_util import bits, error_bound_16, to_dev
 pytestmark = pytest.mark.gpu
 
 SEEN = set()   # kernel families the random cases reached (checked by the last test)
-ALGOS = (ci.ALGO_DEFAULT, ci.ALGO_GENERIC, ci.ALGO_TILE, ci.ALGO_SMALL, ci.ALGO_SKINNY)
+ALGOS = (ci.ALGO_DEFAULT, ci.ALGO_GENERIC, ci.ALGO_TILE, ci.ALGO_SMALL, ci.ALGO_SKINNY, ci.ALGO_MFMA_ANY)
 
 
 def each_family(handle, call):
