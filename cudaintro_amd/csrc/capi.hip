@@ -144,10 +144,12 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->last_error[0] = '\0';
   ctx->ws_partial_bytes = (size_t)64 << 20;
   ctx->ws_counter_bytes = (size_t)64 << 10;
+  ctx->ws_swap_bytes = (size_t)8 << 20;  // 128 bytes per column: N <= 65536
   ctx->workspace = nullptr;
-  if (hipMalloc(&ctx->workspace, ctx->ws_partial_bytes + ctx->ws_counter_bytes) != hipSuccess ||
+  if (hipMalloc(&ctx->workspace,
+                ctx->ws_partial_bytes + ctx->ws_counter_bytes + ctx->ws_swap_bytes) != hipSuccess ||
       hipMemset(static_cast<char*>(ctx->workspace) + ctx->ws_partial_bytes, 0,
-                ctx->ws_counter_bytes) != hipSuccess) {
+                ctx->ws_counter_bytes + ctx->ws_swap_bytes) != hipSuccess) {
     (void)hipGetLastError();
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     delete ctx;

@@ -29,10 +29,12 @@ struct cigemmContext {
   char pending_error[160];
   int algo;  // cigemmAlgo_t; -1 = choose by shape
   // Device scratch of the split-K kernels, allocated once at create: `ws_partial_bytes` of
-  // partial sums followed by `ws_counter_bytes` of arrival counters (zero between calls).
+  // partial sums followed by `ws_counter_bytes` of arrival counters and `ws_swap_bytes` of
+  // exchange words for two K ranges (both zero between calls).
   void* workspace;
   size_t ws_partial_bytes;
   size_t ws_counter_bytes;
+  size_t ws_swap_bytes;
   char last_error[256];
 };
 

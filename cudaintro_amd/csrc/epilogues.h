@@ -53,6 +53,10 @@ struct EpiStore16x4 {
                                              float v3) const {
     *reinterpret_cast<u32x2*>(C + r * ldc + c) = pack(r, c, v0, v1, v2, v3);
   }
+  // two columns (c even): one 4-byte store
+  __device__ __forceinline__ void pair(int64_t r, int64_t c, float v0, float v1) const {
+    *reinterpret_cast<uint32_t*>(C + r * ldc + c) = E16::narrow2(v0, v1);
+  }
   __device__ __forceinline__ void side(int64_t, int64_t, float, float, float, float) const {}
   EpiStore16x4 shift_cols(int64_t c0) const { return EpiStore16x4{C + c0, ldc}; }
 };

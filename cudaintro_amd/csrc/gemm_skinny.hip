@@ -607,7 +607,7 @@ template <typename Math, typename Epi, int XR, int COLS>
 __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
     int M, int N, int stages_per_split, int splits, const char* __restrict__ X, int64_t ldx,
     const char* __restrict__ W, int64_t ldw, Epi epi, uint64_t* __restrict__ partials,
-    uint32_t* __restrict__ counters) {
+    uint32_t* __restrict__ counters, uint64_t* __restrict__ swap_words) {
   typedef KN16KW<XR, COLS> G;
   typedef tile::lds_i16x4 lds_i16x4;
   constexpr int NS = G::NSTAGES, DIST = NS - 1;
@@ -715,7 +715,42 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
     }
     return;
   }
-  // ---- K ranges meet: same exchange as in skinny_kernel (partials as agent-scope 64-bit words,
+  // ---- two K ranges meet through one atomic exchange per 64-bit word.  The word of (slab,
+  // word, thread) is zero between calls; each of the two workgroups swaps its pair of partial
+  // sums in.  The one that gets zero back was first and is done: its pair now waits in the
+  // word.  The one that gets a pair back has both, writes the two outputs and puts the zero
+  // back.  The data travels inside the atomic operation itself, so nothing else has to be
+  // ordered: no partial tile in memory, no counter, no wait, one trip to the coherence point
+  // instead of three.  Which workgroup finishes a word may differ from word to word; a + b is
+  // the same bits either way, and the sum is formed as (0 + range 0) + range 1 like the
+  // reduction below.  A pair of two +0.0f would look like the empty word: it travels as two
+  // -0.0f, which 0 + x turns back into +0.0f.
+  if (splits == 2 && swap_words) {
+    if (m < M) {
+      uint64_t* word = swap_words + ((int64_t)slab * G::PART_WORDS) * 256 + t;
+      uint64_t got[2 * QUADS];
+#pragma unroll
+      for (int p = 0; p < 2 * QUADS; ++p) {
+        uint64_t mine = (uint64_t)__builtin_bit_cast(uint32_t, sum[2 * p]) |
+                        ((uint64_t)__builtin_bit_cast(uint32_t, sum[2 * p + 1]) << 32);
+        if (mine == 0) mine = 0x8000000080000000ull;
+        got[p] = __hip_atomic_exchange(word + 256 * p, mine, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+      }
+#pragma unroll
+      for (int p = 0; p < 2 * QUADS; ++p) {
+        if (got[p] == 0) continue;
+        const float o0 = __builtin_bit_cast(float, (uint32_t)got[p]);
+        const float o1 = __builtin_bit_cast(float, (uint32_t)(got[p] >> 32));
+        const float a0 = split == 0 ? sum[2 * p] : o0, b0 = split == 0 ? o0 : sum[2 * p];
+        const float a1 = split == 0 ? sum[2 * p + 1] : o1, b1 = split == 0 ? o1 : sum[2 * p + 1];
+        epi.pair(m, n0 + c + 2 * p, (0.0f + a0) + b0, (0.0f + a1) + b1);
+        __hip_atomic_store(word + 256 * p, (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    return;
+  }
+  // ---- more K ranges: same exchange as in skinny_kernel (partials as agent-scope 64-bit words,
   // laid out [split][slab][word][thread]; the last workgroup of the slab sums in split order)
   const int slabs = gridDim.x / splits;
   auto part = [&](int sp) {
@@ -779,7 +814,13 @@ void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, 
                      static_cast<const char*>(X), ldx_bytes, static_cast<const char*>(W),
                      ldw_bytes, epi, static_cast<uint64_t*>(ctx->workspace),
                      reinterpret_cast<uint32_t*>(static_cast<char*>(ctx->workspace) +
-                                                 ctx->ws_partial_bytes));
+                                                 ctx->ws_partial_bytes),
+                     // one exchange word per pair of columns and row of x: 128 bytes per column
+                     (size_t)N * 128 <= ctx->ws_swap_bytes
+                         ? reinterpret_cast<uint64_t*>(static_cast<char*>(ctx->workspace) +
+                                                       ctx->ws_partial_bytes +
+                                                       ctx->ws_counter_bytes)
+                         : nullptr);
 }
 
 // COLS = 64, one line per weight row, is the only width in use.  Two lines per row (128-column
@@ -912,9 +953,11 @@ namespace {
 constexpr size_t kStaticPartialBytes = (size_t)16 << 20;  // covers every N <= kStaticMaxN
 constexpr size_t kStaticCounterBytes = 4096;
 constexpr int64_t kStaticMaxN = 16384;
+constexpr size_t kStaticSwapBytes = (size_t)kStaticMaxN * 128;  // exchange words of two K ranges
 constexpr int kStaticMaxDevices = 64;
 
-static __device__ __align__(256) unsigned char scratch[kStaticPartialBytes + kStaticCounterBytes];
+static __device__ __align__(256) unsigned char
+    scratch[kStaticPartialBytes + kStaticCounterBytes + kStaticSwapBytes];
 
 // `scratch` in host code is only a handle for the runtime's symbol table, not a device
 // address: the address of each device's copy is looked up once, with that device current.
@@ -955,9 +998,11 @@ cigemmStatus_t static_device_setup(int dev, StaticDevice** out) {
 
 // The arrival counters must be zero when the GEMM kernel starts.  A kernel, not a memset: this
 // call may be recorded into a graph.
-__global__ void clear_counters_kernel(uint32_t* counters, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) counters[i] = 0u;
+__global__ void clear_counters_kernel(uint32_t* counters, int n, uint64_t* swap_words,
+                                      int64_t n_swap_words) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0;
+  for (int64_t j = i; j < n_swap_words; j += (int64_t)gridDim.x * blockDim.x) swap_words[j] = 0;
 }
 
 cigemmStatus_t static_fail(char* err, size_t err_len, cigemmStatus_t st, const char* fmt, ...)
@@ -998,7 +1043,7 @@ extern "C" cigemmStatus_t cigemm_gemm_bf16_static(void* stream, int64_t M, int64
                        "%s: M=%lld N=%lld beyond the maximum of this entry point (M <= %d, "
                        "N <= %lld: its scratch memory is a fixed %zu-byte device array)",
                        name, (long long)M, (long long)N, XROWS, (long long)kStaticMaxN,
-                       kStaticPartialBytes + kStaticCounterBytes);
+                       kStaticPartialBytes + kStaticCounterBytes + kStaticSwapBytes);
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     (void)hipGetLastError();
@@ -1024,6 +1069,7 @@ extern "C" cigemmStatus_t cigemm_gemm_bf16_static(void* stream, int64_t M, int64
   ctx.workspace = sd->ptr;
   ctx.ws_partial_bytes = kStaticPartialBytes;
   ctx.ws_counter_bytes = kStaticCounterBytes;
+  ctx.ws_swap_bytes = kStaticSwapBytes;
   typedef GeoKN16<tile::MathBF16> GB;
   if (!skinny_shape_ok<GB>(&ctx, M, N, K, 2, A, lda, B, ldb) || ldc % 4 || ((uintptr_t)C & 7))
     return static_fail(err, err_len, CIGEMM_STATUS_NOT_SUPPORTED,
@@ -1031,10 +1077,17 @@ extern "C" cigemmStatus_t cigemm_gemm_bf16_static(void* stream, int64_t M, int64
                        "4, A and B 16-byte and C 8-byte aligned (M=%lld N=%lld K=%lld)",
                        name, (long long)M, (long long)N, (long long)K);
   {
-    // every arrival counter either kernel may use (one per 64-column slab at most)
+    // every arrival counter either kernel may use (one per 64-column slab at most) and the
+    // exchange words of two K ranges (128 bytes per column)
     const int slabs = (int)((N + 63) / 64);
-    hipLaunchKernelGGL(clear_counters_kernel, dim3((slabs + 255) / 256), dim3(256), 0, ctx.stream,
-                       reinterpret_cast<uint32_t*>(sd->ptr + kStaticPartialBytes), slabs);
+    const int64_t words = (int64_t)slabs * 64 * 16;
+    const int blocks = (int)((words / 4 + 255) / 256) > (slabs + 255) / 256
+                           ? (int)((words / 4 + 255) / 256) : (slabs + 255) / 256;
+    hipLaunchKernelGGL(clear_counters_kernel, dim3(blocks), dim3(256), 0, ctx.stream,
+                       reinterpret_cast<uint32_t*>(sd->ptr + kStaticPartialBytes), slabs,
+                       reinterpret_cast<uint64_t*>(sd->ptr + kStaticPartialBytes +
+                                                   kStaticCounterBytes),
+                       words);
   }
   (void)launch_skinny_16_on<tile::MathBF16, BF16>(&ctx, M, N, K, A, lda, B, ldb, C, ldc, true);
   if (ctx.pending_error[0]) {

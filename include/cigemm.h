@@ -185,8 +185,8 @@ CIGEMM_API cigemmStatus_t cigemm_gemm_i8_dequant(
  * No counterpart in the reference.  It is for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid it; creating a
  * handle allocates its workspace).  Same kernel and same results, bit for bit, as
- * cigemm_gemm_bf16 on the same arguments; the kernel's scratch memory (split-K partial sums
- * and arrival counters) is a fixed device array of 16 MiB + 4 KiB inside the library, which
+ * cigemm_gemm_bf16 on the same arguments; the kernel's scratch memory (split-K partial sums,
+ * arrival counters and exchange words) is a fixed device array of 18 MiB + 4 KiB inside the library, which
  * every GPU the process uses holds until the process ends.
  *   Limits: 1 <= M <= 32, N <= 16384, N % 256 == 0, K % 32 == 0, lda and ldb multiples of 8,
  *   ldc a multiple of 4, A and B 16-byte aligned, C 8-byte aligned; anything else returns

@@ -211,3 +211,32 @@ def test_skinny_16bit_both_kernels_exact_inputs(handle, torch_gpu, oracle, rng, 
         got = bits(torch, out)
         np.testing.assert_array_equal(got[:M], want)
         assert (got[M:] == narrow(np.float32(7.0))).all()
+
+
+@pytest.mark.parametrize("zero_part", ["all", "first_range", "second_range", "columns"])
+def test_two_range_exchange_with_zero_partial_sums(handle, torch_gpu, oracle, rng, zero_part):
+    """N = 8192 gives the 64-column kernel two K ranges per slab, which meet through one atomic
+    exchange per pair of outputs; a pair of +0.0 partial sums looks like the exchange word's empty
+    state and travels as -0.0.  Weights that are zero over a whole K range, over everything, or
+    in some columns give such pairs; the results must equal the CPU loop's bits (+0.0 where the
+    sum is zero), three calls in a row (every word returns to empty)."""
+    torch = torch_gpu
+    M, N, K = 3, 8192, 8192
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    X, W = rng.choice(vals, size=(M, K)), rng.choice(vals, size=(K, N))
+    W[rng.random(size=W.shape) < 0.5] = 0
+    if zero_part == "all":
+        W[:] = 0
+    elif zero_part == "first_range":
+        W[:K // 2] = 0
+    elif zero_part == "second_range":
+        W[K // 2:] = 0
+    else:
+        W[:, ::3] = 0
+        W[:, 1000:1100] = 0
+    want = oracle.f32_to_bf16(oracle.gemm_f32(X, W))
+    x, w = to_dev(torch, oracle.f32_to_bf16(X), "bf16"), to_dev(torch, oracle.f32_to_bf16(W), "bf16")
+    for _ in range(3):
+        y = handle.gemm_bf16(x, w)
+        assert handle.last_kernel == "bf16_skinny_32x64_kwaves", handle.last_kernel
+        np.testing.assert_array_equal(bits(torch, y), want)
