@@ -584,20 +584,23 @@ bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, cons
 // the x piece [XR m][16 k] (XR x 32 bytes of the slot, XR = 8, 16 or 32, the smallest that holds
 // M; one DMA instruction of 2 M lanes fills its first M rows), in a ring of NSTAGES slots private
 // to the wave.
-template <int XR_, int COLS_>
+template <int EB_, int XR_, int COLS_>
 struct KN16KW {
-  static constexpr int BN = COLS_;                     // 32 (half a line per weight row), 64, 128
-  static constexpr int K_STAGE = 64;                   // k rows per stage and workgroup
+  static constexpr int EB = EB_;                       // bytes per element: 2 (fp16, bf16) or 1 (int8)
+  static constexpr int BN = COLS_;                     // 16-bit: 64 (one line per weight row; 32 and
+                                                       // 128 were measured); int8: 128 (one line)
+  static constexpr int KW = 32 / EB;                   // k rows per wave and stage = one MFMA's k
+  static constexpr int K_STAGE = 4 * KW;               // k rows per stage and workgroup
   static constexpr int XR = XR_;
-  static constexpr int ROW_BYTES = 2 * BN;
-  static constexpr int W_BYTES = 16 * ROW_BYTES;       // per wave and stage
+  static constexpr int ROW_BYTES = EB * BN;
+  static constexpr int W_BYTES = KW * ROW_BYTES;       // per wave and stage
   static constexpr int W_DMAS = W_BYTES / 1024;        // one instruction moves 1 KiB of whole rows
-  static constexpr int X_BYTES = XR * 32;
+  static constexpr int X_BYTES = XR * 32;              // 32 bytes of k per row of x
   static constexpr int SLOT_BYTES = W_BYTES + X_BYTES;
-  static constexpr int NSTAGES = BN == 32 ? 16 : BN == 64 ? 12 : 7;
+  static constexpr int NSTAGES = W_BYTES == 1024 ? 16 : W_BYTES == 2048 ? 12 : 7;
   static constexpr int DPS = W_DMAS + 1;               // DMA instructions per wave and stage
   static constexpr int WAVE_BYTES = NSTAGES * SLOT_BYTES;
-  static constexpr int RED_LD = BN + 4;                // floats per row of the reduction tiles
+  static constexpr int RED_LD = BN + 4;                // words per row of the reduction tiles
   static constexpr int RED_BYTES = 4 * 32 * RED_LD * 4;
   static constexpr int LDS_BYTES = 4 * WAVE_BYTES > RED_BYTES ? 4 * WAVE_BYTES : RED_BYTES;
   static constexpr int PART_WORDS = BN / 16;           // 64-bit words per thread of a partial tile
@@ -608,20 +611,24 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
     int M, int N, int stages_per_split, int splits, const char* __restrict__ X, int64_t ldx,
     const char* __restrict__ W, int64_t ldw, Epi epi, uint64_t* __restrict__ partials,
     uint32_t* __restrict__ counters, uint64_t* __restrict__ swap_words) {
-  typedef KN16KW<XR, COLS> G;
+  typedef KN16KW<Math::ELEM_BYTES, XR, COLS> G;
   typedef tile::lds_i16x4 lds_i16x4;
+  typedef tile::lds_i32x2 lds_i32x2;
+  typedef typename Math::scalar_t scalar_t;           // float, or int32_t for int8
+  constexpr int EB = G::EB;
   constexpr int NS = G::NSTAGES, DIST = NS - 1;
   constexpr int NT = COLS / 32;                       // 32-column tiles of the slab
   constexpr int PIECES = G::ROW_BYTES / 16;           // 16-byte pieces of a slab row
   constexpr int ROWS_PER_DMA = 64 / PIECES;
-  constexpr int QUADS = COLS / 32;                    // float4 groups per thread of the reduction
+  constexpr int QUADS = COLS / 32;                    // groups of 4 columns per thread of the reduction
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   __shared__ int is_last;
   const int t = threadIdx.x, l = t & 63;
   const int w = __builtin_amdgcn_readfirstlane(t >> 6);
   const int slab = blockIdx.x / splits, split = blockIdx.x % splits;
   const int64_t n0 = (int64_t)slab * G::BN;
-  const int64_t k0 = (int64_t)split * stages_per_split * G::K_STAGE + 16 * w;  // this wave's rows
+  // this wave's k rows of the first stage of the range
+  const int64_t k0 = (int64_t)split * stages_per_split * G::K_STAGE + G::KW * w;
   const int KTS = stages_per_split;
   char* const wave_lds = lds + w * G::WAVE_BYTES;
   const uint32_t wave_base =
@@ -631,14 +638,14 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   // of the x instruction: row l / 2, piece l % 2, lanes of rows below M only (the rows of the
   // slot past M keep whatever the LDS held: an output row depends on its own row of x alone, and
   // rows >= M are never stored)
-  const char* w_src = W + (k0 + l / PIECES) * ldw + n0 * 2 + ((l % PIECES) << 4);
-  const char* x_src = X + (int64_t)(l >> 1) * ldx + k0 * 2 + ((l & 1) << 4);
+  const char* w_src = W + (k0 + l / PIECES) * ldw + n0 * EB + ((l % PIECES) << 4);
+  const char* x_src = X + (int64_t)(l >> 1) * ldx + k0 * EB + ((l & 1) << 4);
   auto issue = [&](int st, int slot) {
     const uint32_t dst = wave_base + slot * G::SLOT_BYTES;
     const char* ws = w_src + (int64_t)st * G::K_STAGE * ldw;
 #pragma unroll
     for (int i = 0; i < G::W_DMAS; ++i) dma16(ws + (int64_t)(ROWS_PER_DMA * i) * ldw, dst + 1024 * i);
-    if (l < 2 * M) dma16(x_src + st * (G::K_STAGE * 2), dst + G::W_BYTES);
+    if (l < 2 * M) dma16(x_src + st * (G::K_STAGE * EB), dst + G::W_BYTES);
   };
 
   typename Math::acc_t acc[NT];
@@ -650,12 +657,15 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   for (int st = 0; st < DIST; ++st)
     if (st < KTS) issue(st, st);
 
-  // fragment addresses within a slot: the transposing read of the W piece (within 16 lanes, lane
-  // i supplies 8 bytes of row i / 4 and receives the k-values of column i; lanes 32-63 take rows
-  // 8-15), and 16 bytes of row l % XR of the x piece
-  const int frag_k = 8 * (l >> 5) + ((l & 15) >> 2);
-  const int frag_n = 16 * ((l >> 4) & 1) + 4 * (l & 3);
-  const int w_off = frag_k * G::ROW_BYTES + frag_n * 2;
+  // fragment addresses within a slot: the transposing read of the W piece (16-bit: within 16
+  // lanes, lane i supplies 8 bytes of row i / 4 and receives the 4 k-values of column i, lanes
+  // 32-63 take rows 8-15, a second read the rows 4 further on; bytes: row i / 2, 8 k-values,
+  // lanes 32-63 rows 16-31, the second read the rows 8 further on), and 16 bytes of row
+  // l % XR of the x piece
+  const int w_off = EB == 2 ? (8 * (l >> 5) + ((l & 15) >> 2)) * G::ROW_BYTES +
+                                  (16 * ((l >> 4) & 1) + 4 * (l & 3)) * 2
+                            : (16 * (l >> 5) + ((l & 15) >> 1)) * G::ROW_BYTES +
+                                  16 * ((l >> 4) & 1) + 8 * (l & 1);
   const int x_off = G::W_BYTES + (l & (XR - 1)) * 32 + ((l >> 5) << 4);
   int slot = 0, dma_slot = DIST;
   for (int s = 0; s < KTS; ++s) {
@@ -669,11 +679,20 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
     const u32x4 xf = *reinterpret_cast<const u32x4*>(sl + x_off);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-      const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(sl + w_off + 64 * j));
-      const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (lds_i16x4*)(sl + w_off + 64 * j + 4 * G::ROW_BYTES));
-      const u32x4 wf = __builtin_shufflevector(__builtin_bit_cast(u32x2, lo),
-                                               __builtin_bit_cast(u32x2, hi), 0, 1, 2, 3);
+      u32x4 wf;
+      if constexpr (EB == 2) {
+        const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(sl + w_off + 64 * j));
+        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_i16x4*)(sl + w_off + 64 * j + 4 * G::ROW_BYTES));
+        wf = __builtin_shufflevector(__builtin_bit_cast(u32x2, lo), __builtin_bit_cast(u32x2, hi),
+                                     0, 1, 2, 3);
+      } else {
+        const i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(sl + w_off + 32 * j));
+        const i32x2 hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+            (lds_i32x2*)(sl + w_off + 32 * j + 8 * G::ROW_BYTES));
+        wf = __builtin_shufflevector(__builtin_bit_cast(u32x2, lo), __builtin_bit_cast(u32x2, hi),
+                                     0, 1, 2, 3);
+      }
       acc[j] = Math::mfma(wf, xf, acc[j]);
     }
     slot = slot + 1 == NS ? 0 : slot + 1;
@@ -682,30 +701,35 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   __syncthreads();  // every wave done with its ring (nothing is in flight): reuse it
 
   // acc[j][4 q + e] = this wave's part of y[l % 32][n0 + 32 j + 8 q + 4 (l / 32) + e]
-  float* red = reinterpret_cast<float*>(lds);  // [4 waves][32 m][RED_LD]
+  scalar_t* red = reinterpret_cast<scalar_t*>(lds);  // [4 waves][32 m][RED_LD]
 #pragma unroll
   for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const f32x4 v = {acc[j][4 * q], acc[j][4 * q + 1], acc[j][4 * q + 2], acc[j][4 * q + 3]};
-      *reinterpret_cast<f32x4*>(red + (w * 32 + (l & 31)) * G::RED_LD + 32 * j + 8 * q +
-                                4 * (l >> 5)) = v;
+      scalar_t* dst = red + (w * 32 + (l & 31)) * G::RED_LD + 32 * j + 8 * q + 4 * (l >> 5);
+      const u32x4 v = {__builtin_bit_cast(uint32_t, (scalar_t)acc[j][4 * q]),
+                       __builtin_bit_cast(uint32_t, (scalar_t)acc[j][4 * q + 1]),
+                       __builtin_bit_cast(uint32_t, (scalar_t)acc[j][4 * q + 2]),
+                       __builtin_bit_cast(uint32_t, (scalar_t)acc[j][4 * q + 3])};
+      *reinterpret_cast<u32x4*>(dst) = v;
     }
   __syncthreads();
   // thread t: row t / 8, columns 4 QUADS (t % 8) .. + 4 QUADS - 1, summed over the waves in
   // wave order
   const int m = t >> 3, c = (t & 7) * 4 * QUADS;
-  float sum[4 * QUADS];
+  scalar_t sum[4 * QUADS];
 #pragma unroll
   for (int h = 0; h < QUADS; ++h) {
-    f32x4 v = *reinterpret_cast<const f32x4*>(red + m * G::RED_LD + c + 4 * h);
 #pragma unroll
-    for (int ww = 1; ww < 4; ++ww) {
-      const f32x4 p = *reinterpret_cast<const f32x4*>(red + (ww * 32 + m) * G::RED_LD + c + 4 * h);
-      v += p;
+    for (int ww = 0; ww < 4; ++ww) {
+      const u32x4 p = *reinterpret_cast<const u32x4*>(red + (ww * 32 + m) * G::RED_LD + c + 4 * h);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t bits = p[e];
+        const scalar_t v = __builtin_bit_cast(scalar_t, bits);
+        sum[4 * h + e] = ww == 0 ? v : sum[4 * h + e] + v;
+      }
     }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) sum[4 * h + e] = v[e];
   }
   if (splits == 1) {
     if (m < M) {
@@ -725,6 +749,7 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   // the same bits either way, and the sum is formed as (0 + range 0) + range 1 like the
   // reduction below.  A pair of two +0.0f would look like the empty word: it travels as two
   // -0.0f, which 0 + x turns back into +0.0f.
+  if constexpr (EB == 2) {
   if (splits == 2 && swap_words) {
     if (m < M) {
       uint64_t* word = swap_words + ((int64_t)slab * G::PART_WORDS) * 256 + t;
@@ -750,6 +775,7 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
     }
     return;
   }
+  }
   // ---- more K ranges: same exchange as in skinny_kernel (partials as agent-scope 64-bit words,
   // laid out [split][slab][word][thread]; the last workgroup of the slab sums in split order)
   const int slabs = gridDim.x / splits;
@@ -772,13 +798,13 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   __syncthreads();
   if (!is_last) return;
   if (m < M) {
-    float q4[QUADS][4];
+    scalar_t q4[QUADS][4];
     const int64_t stride = (int64_t)slabs * G::PART_WORDS * 256;
     switch (splits) {
-      case 2: sum_partials<float, QUADS, 2>(part(0), stride, q4); break;
-      case 4: sum_partials<float, QUADS, 4>(part(0), stride, q4); break;
-      case 8: sum_partials<float, QUADS, 8>(part(0), stride, q4); break;
-      default: sum_partials<float, QUADS, 16>(part(0), stride, q4); break;
+      case 2: sum_partials<scalar_t, QUADS, 2>(part(0), stride, q4); break;
+      case 4: sum_partials<scalar_t, QUADS, 4>(part(0), stride, q4); break;
+      case 8: sum_partials<scalar_t, QUADS, 8>(part(0), stride, q4); break;
+      default: sum_partials<scalar_t, QUADS, 16>(part(0), stride, q4); break;
     }
 #pragma unroll
     for (int h = 0; h < QUADS; ++h) epi(m, n0 + c + 4 * h, q4[h][0], q4[h][1], q4[h][2], q4[h][3]);
@@ -802,7 +828,7 @@ inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, 
 template <typename Math, typename Epi, int XR, int COLS>
 void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
                            int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
-  typedef KN16KW<XR, COLS> G;
+  typedef KN16KW<Math::ELEM_BYTES, XR, COLS> G;
   static_assert(G::LDS_BYTES + 64 <= 160 * 1024, "rings and the arrival flag must fit the LDS");
   auto kern = skinny_kn16_kwaves_kernel<Math, Epi, XR, COLS>;
   static std::atomic<uint64_t> lds_set{0};
@@ -910,10 +936,48 @@ bool launch_skinny_16(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64
   return true;
 }
 
+// int8 K x N weights: the K-over-the-waves kernel of the 16-bit types with 128-column slabs (one
+// 128-byte line per weight row) and 128 k per stage; N and K multiples of 128.  Other shapes go
+// to the tile kernel (64-row tiles, split-K).
+struct SlabKN8 {
+  static constexpr int BN = 128, K_ELEMS = 128;
+};
+static bool launch_skinny_i8_kn(cigemmContext* ctx, int64_t M, int64_t N, int64_t K,
+                                const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb,
+                                int32_t* C, int64_t ldc, const DequantArgs* dq) {
+  if (!skinny_shape_ok<SlabKN8>(ctx, M, N, K, 1, A, lda, B, ldb)) return false;
+  if ((size_t)(N / SlabKN8::BN) * 4 > ctx->ws_counter_bytes) return false;
+  if (!dq) {
+    if (ldc % 4 || ((uintptr_t)C & 15)) return false;
+    launch_kn16_kwaves<tile::MathI8, 128>(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32x4{C, ldc});
+    ctx->last_kernel = "i8_skinny_32x128_kwaves_kn";
+    return true;
+  }
+  if (dq->out_bf16 ? (dq->ldo % 4 || ((uintptr_t)dq->out & 7))
+                   : (dq->ldo % 4 || ((uintptr_t)dq->out & 15)))
+    return false;
+  if (dq->sb_vec && ((uintptr_t)dq->sb & 15)) return false;
+  if (dq->acc_out && (dq->ldacc % 4 || ((uintptr_t)dq->acc_out & 15))) return false;
+#define CIG_DQ(OB, DA)                                                                          \
+  launch_kn16_kwaves<tile::MathI8, 128>(ctx, M, N, K, A, lda, B, ldb,                            \
+                                        EpiDequantX4<OB, DA>{dq->out, dq->ldo, dq->sa, dq->sb,   \
+                                                             dq->sa_vec, dq->sb_vec,             \
+                                                             dq->acc_out, dq->ldacc})
+  const bool dump = dq->acc_out != nullptr;
+  if (dq->out_bf16) {
+    if (dump) CIG_DQ(true, true); else CIG_DQ(true, false);
+  } else {
+    if (dump) CIG_DQ(false, true); else CIG_DQ(false, false);
+  }
+#undef CIG_DQ
+  ctx->last_kernel = "i8_skinny_32x128_kwaves_kn_dequant";
+  return true;
+}
+
 bool launch_skinny_i8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
                       int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
                       int64_t ldc, const DequantArgs* dq) {
-  if (!b_nk) return false;  // K x N int8 weights at M <= 32 go to the tile kernel (64-row tiles)
+  if (!b_nk) return launch_skinny_i8_kn(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
   if (!skinny_shape_ok<Slab32>(ctx, M, N, K, 1, A, lda, B, ldb)) return false;
   if (!dq) {
     if (ldc % 4 || ((uintptr_t)C & 15)) return false;

@@ -240,3 +240,34 @@ def test_two_range_exchange_with_zero_partial_sums(handle, torch_gpu, oracle, rn
         y = handle.gemm_bf16(x, w)
         assert handle.last_kernel == "bf16_skinny_32x64_kwaves", handle.last_kernel
         np.testing.assert_array_equal(bits(torch, y), want)
+
+
+@pytest.mark.parametrize("M", [1, 5, 8, 16, 17, 32])
+@pytest.mark.parametrize("N,K", [(128, 128), (1024, 512), (8192, 8192), (256, 4096 + 128), (2048, 1024),
+                                 (8192 + 128, 1024 + 128)])
+def test_skinny_int8_kn(handle, torch_gpu, oracle, rng, M, N, K):
+    """int8 K x N weights at M <= 32: the K-over-the-waves kernel with 128-column slabs, one to
+    sixteen K ranges per slab; raw accumulators (into a guarded buffer, twice) and both
+    dequantized output types, bit for bit."""
+    torch = torch_gpu
+    X = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    W = rng.integers(-127, 128, size=(K, N), dtype=np.int8)
+    acc_ref = oracle.gemm_i8_i32(X, W, b_is_nk=False)
+    xd, wd = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda()
+    out = torch.full((M + 2, N + 4), -9, dtype=torch.int32, device="cuda")
+    for _ in range(2):
+        handle.gemm_i8_i32(xd, wd, ci.B_KN, out=out[:M, :N])
+        assert handle.last_kernel == "i8_skinny_32x128_kwaves_kn", handle.last_kernel
+        o = out.cpu().numpy()
+        np.testing.assert_array_equal(o[:M, :N], acc_ref)
+        assert (o[M:] == -9).all() and (o[:, N:] == -9).all()
+    sa = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
+    sb = rng.uniform(1e-3, 5e-2, N).astype(np.float32)
+    for out_type, ot in (("f32", ci.OUT_F32), ("bf16", ci.OUT_BF16)):
+        y, acc = handle.gemm_i8_dequant(xd, wd, torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda(),
+                                        ci.B_KN, ot, dump_acc=True)
+        assert handle.last_kernel == "i8_skinny_32x128_kwaves_kn_dequant", handle.last_kernel
+        np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
+        expect = oracle.dequant(acc_ref, sa, sb, out_dtype=out_type, sa_per_row=M > 1, sb_per_col=True)
+        got = bits(torch, y) if out_type == "bf16" else y.cpu().numpy()
+        np.testing.assert_array_equal(got, expect)
