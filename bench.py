@@ -434,6 +434,21 @@ def main():
         per_config[f"bf16_{n}"] = {"tflops": achieved, "frac_of_peak": achieved / PEAK_16BIT_TFLOPS,
                                    "peak": PEAK_16BIT_TFLOPS, "ms": ev / args.steps * 1e3,
                                    "kernel": kernel}
+        # the same for fp32: every dimension odd
+        Mx, Nx, Kx = 4095, 4097, 4099
+        a = torch.from_numpy(np.random.Generator(np.random.PCG64(5)).uniform(-1, 1, (Mx, Kx)).astype(np.float32)).cuda()
+        b = torch.from_numpy(np.random.Generator(np.random.PCG64(6)).uniform(-1, 1, (Kx, Nx)).astype(np.float32)).cuda()
+        c = torch.empty((Mx, Nx), dtype=torch.float32, device="cuda")
+        w, e = time_calls(torch, lambda: handle.gemm_f32(a, b, out=c), 10, 3)
+        name_a = handle.last_kernel
+        with handle.algo(ci.ALGO_GENERIC):
+            w, e_s = time_calls(torch, lambda: handle.gemm_f32(a, b, out=c), 3, 1)
+        t = wl.gemm_ops(Mx, Nx, Kx) * 10 / e / 1e12
+        per_config[f"fp32_{Mx}x{Nx}x{Kx}_unaligned"] = {
+            "tflops": t, "frac_of_peak": t / PEAK_FP32_MATRIX_TFLOPS, "peak": PEAK_FP32_MATRIX_TFLOPS,
+            "ms": e / 10 * 1e3, "kernel": name_a,
+            "scalar_kernel_tflops": wl.gemm_ops(Mx, Nx, Kx) * 3 / e_s / 1e12}
+        del a, b, c
 
         def run_i8(name, M, N, K, make, dequant):
             log(f"[bench] {name}")

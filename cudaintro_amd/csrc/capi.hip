@@ -229,8 +229,9 @@ static cigemmStatus_t algo_refused(cigemmHandle_t h, const char* name) {
               "%s: the selected kernel family (algo %d) does not take this call", name, h->algo);
 }
 
-// fp32 dispatch.  DEFAULT: one of the two MFMA kernels when the shape allows, else the
-// any-shape kernel.  Returns false when a selected family refuses the call.
+// fp32 dispatch.  DEFAULT: one of the two aligned MFMA kernels when the shape allows, else the
+// any-shape MFMA kernel (the scalar kernel only if its tile grid does not fit a launch).
+// Returns false when a selected family refuses the call.
 static bool dispatch_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K, const float* A,
                          int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
                          const BiasAct* ba) {
@@ -243,13 +244,15 @@ static bool dispatch_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K, cons
       return true;
     case CIGEMM_ALGO_SKINNY:
     case CIGEMM_ALGO_TILE_PAIRED:
-    case CIGEMM_ALGO_MFMA_ANY:
       return false;
+    case CIGEMM_ALGO_MFMA_ANY:
+      return launch_mfma_any_f32(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
     case CIGEMM_ALGO_GENERIC:
       launch_generic_f32(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
       return true;
     default:
-      if (!launch_f32_mfma(h, M, N, K, A, lda, B, ldb, C, ldc, ba))
+      if (!launch_f32_mfma(h, M, N, K, A, lda, B, ldb, C, ldc, ba) &&
+          !launch_mfma_any_f32(h, M, N, K, A, lda, B, ldb, C, ldc, ba))
         launch_generic_f32(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
       return true;
   }

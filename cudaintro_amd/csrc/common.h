@@ -208,11 +208,14 @@ struct DequantArgs {
 void launch_generic_f32(cigemmContext*, int64_t M, int64_t N, int64_t K, const float* A,
                         int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
                         const BiasAct* ba = nullptr);
-// gemm_ragged.hip: any shape, any alignment, on the matrix cores (16-bit and int8).  False when
+// gemm_ragged.hip: any shape, any alignment, on the matrix cores.  False when
 // the tile grid does not fit a launch (nothing launched).
 bool launch_mfma_any_16(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
                         const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                         uint16_t* C, int64_t ldc);
+bool launch_mfma_any_f32(cigemmContext*, int64_t M, int64_t N, int64_t K, const float* A,
+                         int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                         const BiasAct* ba);
 bool launch_mfma_any_i8(cigemmContext*, int64_t M, int64_t N, int64_t K, const int8_t* A,
                         int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
                         int64_t ldc, const DequantArgs* dq);

@@ -34,6 +34,11 @@ bool launch_f32_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const 
         tile_ok && K >= 2048 && one_round &&
         tile::plan_small(ctx, M, N, K * 4, tile::MathF32::STAGE_UNIT_US, K * 4 * N)
                 .splits > 1;
+    // What the tile kernel cannot take (B or C rows not 16-byte aligned, an odd N) and fills the
+    // chip with 128 x 128 tiles is left to the any-shape matrix-core kernel (4096 x 4095 x 4096:
+    // 109 against 63 TFLOP/s; at 1000^3, 64 such tiles, this kernel is 3x the faster one).
+    const double tiles128 = (double)((M + 127) / 128) * (double)((N + 127) / 128);
+    if (!tile_ok && tiles128 >= cus) return false;
     if (!tile_ok || (small_cost < tile_cost && !long_k_split)) {
       launch_f32_small(ctx, M, N, K, A, lda, B, ldb, C, ldc, ba);
       return true;

@@ -1,5 +1,5 @@
-// Any-shape GEMM on the matrix cores, for the 16-bit and int8 calls that the LDS-DMA tile
-// kernel cannot take (an odd N, rows or pointers that are not 16-byte aligned, a K whose bytes
+// Any-shape GEMM on the matrix cores, for the calls that the LDS-DMA tile kernel and the small
+// fp32 kernel cannot take (an odd N, rows or pointers that are not 16-byte aligned, a K whose bytes
 // are not a multiple of 16): the scalar any-shape kernel runs those at a few TFLOP/s, two orders
 // of magnitude below the tile kernel, and the library this path replaces has no such cliff
 // (quantization/GEMM_bf16.cu:51-56 passes whatever m, n, k, lda, ldb it is given).
@@ -22,10 +22,11 @@
 // the scalar any-shape kernel, so every output type and scale mode is served and nothing is
 // assumed about the alignment of C either.
 //
-// Arithmetic: products exact, fp32 (int32) accumulation inside the MFMA in its own order --
-// int8 results equal the CPU loop bit for bit, 16-bit results are within the same K-scaled bound
-// as the tile kernel's.  fp32 calls never come here: the scalar kernel's fp32 results equal the
-// CPU loop bit for bit, which the fp32 tests rely on.
+// Arithmetic: 16-bit and int8 products exact, fp32 (int32) accumulation inside the MFMA in its
+// own order -- int8 results equal the CPU loop bit for bit, 16-bit results are within the same
+// K-scaled bound as the tile kernel's; fp32 (v_mfma_f32_32x32x2_f32: true fp32 products and sums)
+// within the same scaled 1e-5 tolerance of the CPU loop as the fp32 tile kernel's.  Only the
+// scalar kernel (CIGEMM_ALGO_GENERIC) reproduces the CPU loop's fp32 bits.
 #include "common.h"
 #include "mfma_tile.h"
 
@@ -47,6 +48,11 @@ template <>
 struct RaggedElem<1> {
   typedef uint8_t type;
   static constexpr int KN_PITCH = 160;  // [64 k][128 B], 8 consecutive rows 8 banks apart
+};
+template <>
+struct RaggedElem<4> {
+  typedef uint32_t type;                // fp32, moved as bits
+  static constexpr int KN_PITCH = 544;  // [16 k][512 B], rows k and k + 4 half the banks apart
 };
 
 // One 16-byte piece = elements [col, col + CE) of row `row` of a row-major matrix with `rows`
@@ -104,11 +110,11 @@ __global__ __launch_bounds__(256) void mfma_any_kernel(int64_t M, int64_t N, int
   typedef typename E::type elem_t;
   typedef typename Math::acc_t acc_t;
   constexpr int EB = Math::ELEM_BYTES;
-  constexpr int KE = RK / EB;               // elements of k per step: 32 or 64
+  constexpr int KE = RK / EB;               // elements of k per step: 32, 64 or (fp32) 16
   constexpr int CE = 16 / EB;               // elements per 16-byte piece
-  constexpr int KN_PIECES = RT * EB / 16;   // pieces per k row of a K x N tile: 16 or 8
+  constexpr int KN_PIECES = RT * EB / 16;   // pieces per k row of a K x N tile: 16, 8 or 32
   constexpr int BP = E::KN_PITCH;
-  static_assert(RT * RROW == KE * BP, "both B layouts fill the same LDS array");
+  static_assert(RT * RROW >= KE * BP, "both B layouts fit the same LDS array");
   __shared__ __attribute__((aligned(16))) unsigned char As[RT * RROW];
   __shared__ __attribute__((aligned(16))) unsigned char Bs[RT * RROW];
   const elem_t* __restrict__ A = static_cast<const elem_t*>(Av);
@@ -183,6 +189,14 @@ __global__ __launch_bounds__(256) void mfma_any_kernel(int64_t M, int64_t N, int
   auto b_fragment = [&](int j, int kk) -> u32x4 {
     if constexpr (B_NK) {
       return *reinterpret_cast<const u32x4*>(b_frag + 32 * j * RROW + 32 * kk);
+    } else if constexpr (EB == 4) {
+      // four single floats: column n of k rows 8 kk + 4 (l / 32) + e
+      const unsigned char* p = Bs + (8 * kk + 4 * (l >> 5)) * BP + (64 * wn + 32 * j + (l & 31)) * 4;
+      const u32x4 v = {*reinterpret_cast<const uint32_t*>(p),
+                       *reinterpret_cast<const uint32_t*>(p + BP),
+                       *reinterpret_cast<const uint32_t*>(p + 2 * BP),
+                       *reinterpret_cast<const uint32_t*>(p + 3 * BP)};
+      return v;
     } else if constexpr (EB == 2) {
       // an MFMA's 16 k rows start at row 16 kk; the second read takes the rows 4 further on
       const unsigned char* p = b_tr + 16 * kk * BP + 64 * j;
@@ -214,10 +228,22 @@ __global__ __launch_bounds__(256) void mfma_any_kernel(int64_t M, int64_t N, int
           af[i] = *reinterpret_cast<const u32x4*>(a_frag + 32 * i * RROW + 32 * kk);
           bf[i] = b_fragment(i, kk);
         }
+        if constexpr (EB == 4) {
+          // 8 k per 32-byte chunk: the MFMA takes one float per lane and operand (lanes 0-31
+          // k, lanes 32-63 k + 4), so element e of the two fragments feeds MFMA e
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+          for (int e = 0; e < 4; ++e)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) acc[i][j] = Math::mfma(af[i], bf[j], acc[i][j]);
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+              for (int j = 0; j < 2; ++j)
+                acc[i][j] = Math::mfma(Math::afrag(af[i], e), Math::afrag(bf[j], e), acc[i][j]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = Math::mfma(af[i], bf[j], acc[i][j]);
+        }
       }
       __syncthreads();
     }
@@ -291,6 +317,21 @@ bool launch_mfma_any_16(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int
   } else {
     launch_any<tile::MathF16, false>(ctx, M, N, K, A, lda, B, ldb, EpiStore16<F16>{C, ldc});
     ctx->last_kernel = "f16_mfma_any_128x128x32";
+  }
+  return true;
+}
+
+bool launch_mfma_any_f32(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const float* A,
+                         int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                         const BiasAct* ba) {
+  if (!any_shape_ok(M, N)) return false;
+  if (ba) {
+    launch_any<tile::MathF32, false>(ctx, M, N, K, A, lda, B, ldb,
+                                     EpiBiasActF32{C, ldc, ba->bias, ba->relu});
+    ctx->last_kernel = "f32_mfma_any_128x128x16_bias_act";
+  } else {
+    launch_any<tile::MathF32, false>(ctx, M, N, K, A, lda, B, ldb, EpiStoreF32{C, ldc});
+    ctx->last_kernel = "f32_mfma_any_128x128x16";
   }
   return true;
 }

@@ -130,8 +130,8 @@ typedef enum cigemmAlgo {
                               chosen by DEFAULT: it issues more matrix instructions per cycle and
                               is slower on a power-limited chip; kept selectable as the measured
                               counterpart of CIGEMM_ALGO_TILE */
-  CIGEMM_ALGO_MFMA_ANY = 5 /* 16-bit and int8: 128x128 MFMA tiles fed by element-wise, bounds-checked
-                              loads and stores: any shape, leading dimension and alignment.
+  CIGEMM_ALGO_MFMA_ANY = 5 /* 128x128 MFMA tiles fed by bounds-checked loads and stores at element
+                              alignment: any shape, leading dimension and alignment, every type.
                               DEFAULT uses it for what the families above do not take */
 } cigemmAlgo_t;
 CIGEMM_API cigemmStatus_t cigemmSetAlgo(cigemmHandle_t handle, cigemmAlgo_t algo);

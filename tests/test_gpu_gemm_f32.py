@@ -92,7 +92,8 @@ def test_generic_kernel_equals_cpu_loop_bit_for_bit(handle, torch_gpu, oracle, r
     the same order as the reference CPU loop."""
     A = rng.uniform(-1, 1, size=(77, 300)).astype(np.float32)
     B = rng.uniform(-1, 1, size=(300, 91)).astype(np.float32)
-    C = run(handle, torch_gpu, A, B)
+    with handle.algo(ci.ALGO_GENERIC):
+        C = run(handle, torch_gpu, A, B)
     assert "generic" in handle.last_kernel
     np.testing.assert_array_equal(C, oracle.gemm_f32(A, B))
 
@@ -240,7 +241,7 @@ def test_narrow_kernel_weights_inside_a_wider_matrix(handle, torch_gpu, oracle, 
 
 def test_default_choice_by_shape(handle, torch_gpu):
     """Small problems and narrow outputs go to the 32x32 kernel, large ones to 256-column
-    tiles, what neither takes to the any-shape kernel."""
+    tiles, what neither takes to the any-shape matrix-core kernel."""
     torch = torch_gpu
     def kernel_for(M, N, K):
         handle.gemm_f32(torch.zeros((M, K), device="cuda"), torch.zeros((K, N), device="cuda"))
@@ -254,7 +255,7 @@ def test_default_choice_by_shape(handle, torch_gpu):
     assert "x256x16_w" in kernel_for(20000, 512, 784)
     assert kernel_for(512, 512, 4096).endswith("_splitk")      # long K: tile kernel, K split
     assert kernel_for(256, 1024, 8192).endswith("_splitk")
-    assert "generic" in kernel_for(77, 91, 300)
+    assert "mfma_any" in kernel_for(77, 91, 300)
 
 
 def test_all_kernels_agree_on_exact_inputs(handle, torch_gpu, oracle, rng):

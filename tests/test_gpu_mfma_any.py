@@ -100,16 +100,56 @@ def test_any_shape_int8(handle, torch_gpu, oracle, rng, layout, M, N, K):
                 np.testing.assert_array_equal(got, expect)
 
 
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_any_shape_f32(handle, torch_gpu, oracle, rng, M, N, K):
+    """fp32: within the scaled 1e-5 tolerance of the CPU loop on uniform inputs, bit for bit on
+    exact-arithmetic inputs; with and without bias + ReLU."""
+    torch = torch_gpu
+    for exact in (True, False):
+        if exact:
+            A, B = rng.choice(VALS, size=(M, K)), rng.choice(VALS, size=(K, N))
+        else:
+            A = rng.uniform(-1, 1, size=(M, K)).astype(np.float32)
+            B = rng.uniform(-1, 1, size=(K, N)).astype(np.float32)
+        bias = rng.choice(VALS, size=N) if exact else rng.uniform(-1, 1, size=N).astype(np.float32)
+        _, a = embed(torch, A, torch.float32, 1, 3, float("nan"))
+        _, b = embed(torch, B, torch.float32, 3, 1, float("nan"))
+        flat, out = embed(torch, np.zeros((M, N), np.float32), torch.float32, 1, 5, 0.0)
+        for algo in (ci.ALGO_MFMA_ANY, ci.ALGO_DEFAULT):
+            for with_bias in (False, True):
+                flat.fill_(3.0)
+                with handle.algo(algo):
+                    if with_bias:
+                        handle.linear_f32(a, b, torch.from_numpy(bias).cuda(), ci.ACT_RELU, out=out)
+                        cpu = oracle.linear_f32(A, B, bias, True)
+                    else:
+                        handle.gemm_f32(a, b, out=out)
+                        cpu = oracle.gemm_f32(A, B)
+                assert "f32_mfma_any" in handle.last_kernel, handle.last_kernel
+                got = out.cpu().numpy()
+                if exact:
+                    np.testing.assert_array_equal(got, cpu)
+                else:
+                    plain = oracle.gemm_f32(A, B).astype(np.float64)
+                    rms = float(np.sqrt(np.mean(plain ** 2)))
+                    lim = 1e-5 * np.maximum(np.abs(plain), rms) + 1e-30
+                    assert (np.abs(got.astype(np.float64) - cpu) <= lim).all()
+                f = flat.cpu().numpy()
+                guard = np.ones(f.shape, bool)
+                for i in range(M):
+                    guard[1 + i * (N + 5): 1 + i * (N + 5) + N] = False
+                assert (f[guard] == 3.0).all()
+
+
 def test_any_shape_kernel_is_the_fallback_not_the_first_choice(handle, torch_gpu):
-    """Aligned shapes keep the LDS-DMA tile kernel; fp32 never goes to the any-shape MFMA kernel
-    (its scalar kernel equals the CPU loop bit for bit)."""
+    """Aligned shapes keep the LDS-DMA tile kernel and the small fp32 kernel."""
     torch = torch_gpu
     a = torch.zeros((256, 256), dtype=torch.bfloat16, device="cuda")
     handle.gemm_bf16(a, a)
     assert "mfma_any" not in handle.last_kernel and "_mfma_" in handle.last_kernel
-    f = torch.zeros((65, 63), dtype=torch.float32, device="cuda")
-    handle.gemm_f32(f, torch.zeros((63, 61), dtype=torch.float32, device="cuda"))
-    assert "generic" in handle.last_kernel
-    with handle.algo(ci.ALGO_MFMA_ANY):
-        with pytest.raises(ci.CigemmError, match="NOT_SUPPORTED"):
-            handle.gemm_f32(f, torch.zeros((63, 61), dtype=torch.float32, device="cuda"))
+    f = torch.zeros((512, 512), dtype=torch.float32, device="cuda")
+    handle.gemm_f32(f, f)
+    assert "mfma_any" not in handle.last_kernel
+    f = torch.zeros((4096, 64), dtype=torch.float32, device="cuda")
+    handle.gemm_f32(f, torch.zeros((64, 4096), dtype=torch.float32, device="cuda"))
+    assert "x256x16_w" in handle.last_kernel
