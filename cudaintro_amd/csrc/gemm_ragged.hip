@@ -105,7 +105,7 @@ template <typename Math, bool B_NK, typename Epi>
 __global__ __launch_bounds__(256) void mfma_any_kernel(int64_t M, int64_t N, int64_t K,
                                                        const void* __restrict__ Av, int64_t lda,
                                                        const void* __restrict__ Bv, int64_t ldb,
-                                                       Epi epi) {
+                                                       Epi epi, int tiles_m, int tiles_n) {
   typedef RaggedElem<Math::ELEM_BYTES> E;
   typedef typename E::type elem_t;
   typedef typename Math::acc_t acc_t;
@@ -122,7 +122,21 @@ __global__ __launch_bounds__(256) void mfma_any_kernel(int64_t M, int64_t N, int
 
   const int t = threadIdx.x, l = t & 63, w = t >> 6;
   const int wm = w >> 1, wn = w & 1;
-  const int64_t m0 = (int64_t)blockIdx.y * RT, n0 = (int64_t)blockIdx.x * RT;
+  // Workgroups go to the 8 XCDs round-robin; each XCD gets a contiguous range of logical ids,
+  // which walk the tile grid in column-major groups of 8 tile rows: the tiles resident on one
+  // XCD at a time (about three per compute unit) share A and B panels in that XCD's L2.
+  int tm, tn;
+  {
+    constexpr int64_t XCDS = 8, GROUP_M = 8;
+    const int64_t nwg = (int64_t)tiles_m * tiles_n, pid = blockIdx.x;
+    const int64_t xcd = pid % XCDS, local = pid / XCDS, base = nwg / XCDS, rem = nwg % XCDS;
+    const int64_t wg = xcd * base + (xcd < rem ? xcd : rem) + local;
+    const int64_t per_group = GROUP_M * tiles_n, first_m = wg / per_group * GROUP_M;
+    const int64_t gsize = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+    tm = (int)(first_m + wg % per_group % gsize);
+    tn = (int)(wg % per_group / gsize);
+  }
+  const int64_t m0 = (int64_t)tm * RT, n0 = (int64_t)tn * RT;
 
   // 512 pieces per operand and step, two per thread: piece c = t + 256 i.
   // k-contiguous operand: row c / 4, piece c % 4 of its 64 bytes; K x N: k row c / KN_PIECES,
@@ -273,9 +287,9 @@ __global__ __launch_bounds__(256) void mfma_any_kernel(int64_t M, int64_t N, int
 template <typename Math, bool B_NK, typename Epi>
 void launch_any(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
                 const void* B, int64_t ldb, const Epi& epi) {
-  const dim3 grid((unsigned)((N + RT - 1) / RT), (unsigned)((M + RT - 1) / RT), 1);
-  hipLaunchKernelGGL((mfma_any_kernel<Math, B_NK, Epi>), grid, dim3(256), 0, ctx->stream, M, N, K,
-                     A, lda, B, ldb, epi);
+  const int tiles_m = (int)((M + RT - 1) / RT), tiles_n = (int)((N + RT - 1) / RT);
+  hipLaunchKernelGGL((mfma_any_kernel<Math, B_NK, Epi>), dim3((unsigned)(tiles_m * tiles_n)),
+                     dim3(256), 0, ctx->stream, M, N, K, A, lda, B, ldb, epi, tiles_m, tiles_n);
 }
 
 template <bool B_NK>
@@ -300,9 +314,10 @@ void launch_any_i8_layout(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, c
 #undef CIG_DQ
 }
 
-// the grid's y dimension holds the tile rows
+// one workgroup per tile, in a one-dimensional grid
 bool any_shape_ok(int64_t M, int64_t N) {
-  return M > 0 && N > 0 && (M + RT - 1) / RT <= 65535 && (N + RT - 1) / RT <= 2147483647LL;
+  return M > 0 && N > 0 && ((M + RT - 1) / RT) * ((N + RT - 1) / RT) <= 2147483647LL &&
+         (M + RT - 1) / RT <= 2147483647LL && (N + RT - 1) / RT <= 2147483647LL;
 }
 
 }  // namespace
