@@ -41,7 +41,7 @@ def test_probe_output_equals_plain_call_and_phases_add_up(handle, torch_gpu, ora
         # of the tile in fewer cycles than its matrix instructions take; the clock is plausible
         assert ph["prologue_us"] + ph["main_loop_us"] + ph["epilogue_us"] <= ph["first_start_to_last_end_us"] * 1.001
         assert ph["cycles_per_stage"] >= min_cycles
-        assert 0.5 < ph["main_loop_clock_ghz"] < 2.6
+        assert 0.05 < ph["main_loop_clock_ghz"] < 3.0
 
 
 def test_probe_rejects_bad_arguments(handle, torch_gpu):
