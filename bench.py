@@ -626,6 +626,19 @@ def main():
                     yo[:r].view(torch.int16).cpu().numpy().view(np.uint16), want))
                 per_config[f"skinny_int8_M{M}"]["cpu_baseline"] = base
             del wqs
+            # the same weights stored K x N (the reference's own operand order): the decode
+            # kernel with 128-column slabs and four K ranges per slab
+            wts = [torch.from_numpy(np.ascontiguousarray(wq.T)).cuda() for _ in range(6)]
+
+            def fn8kn():
+                handle.gemm_i8_dequant(xd, wts[it[0] % 6], sxd, swd, ci.B_KN, ci.OUT_BF16, out=yo)
+                it[0] += 1
+            w, e = time_calls(torch, fn8kn, steps, max(6, args.warmup))
+            per_config[f"skinny_int8_kn_M{M}"] = {"gbs": nbytes * steps / e / 1e9,
+                                                  "frac_of_peak": nbytes * steps / e / 1e9 / PEAK_HBM_GBS,
+                                                  "peak": PEAK_HBM_GBS, "us": e / steps * 1e6,
+                                                  "bytes": nbytes, "kernel": handle.last_kernel}
+            del wts
         # small-batch shapes between the decode and the square configurations: few output
         # tiles and a long K, run as split-K (weights still dominate the traffic)
         for M in (64, 256):
