@@ -1,7 +1,7 @@
 // Any-shape GEMM on the matrix cores, for the calls that the LDS-DMA tile kernel and the small
 // fp32 kernel cannot take (an odd N, rows or pointers that are not 16-byte aligned, a K whose bytes
-// are not a multiple of 16): the scalar any-shape kernel runs those at a few TFLOP/s, two orders
-// of magnitude below the tile kernel, and the library this path replaces has no such cliff
+// are not a multiple of 16): the scalar any-shape kernel runs those at 30 (16-bit) to 45 (fp32)
+// TFLOP/s, far below the tile kernel, and the library this path replaces has no such cliff
 // (quantization/GEMM_bf16.cu:51-56 passes whatever m, n, k, lda, ldb it is given).
 //
 // One 128 x 128 output tile per 256-thread workgroup, four waves of 64 x 64 (2 x 2 MFMA tiles
@@ -13,11 +13,12 @@
 // would keep the loads from overlapping the multiplies).  The pieces are held in registers
 // while the previous step multiplies, and written to LDS as the rows
 // they are: A, and B when it is N x K, as [row][64 B of k] with rows 80 bytes apart; a K x N
-// operand as [k][128 columns] with rows 320 (16-bit) or 160 (int8) bytes apart.  MFMA operands
+// operand as [k][128 columns] with rows 320 (16-bit), 160 (int8) or 544 (fp32) bytes apart.  MFMA operands
 // of the first kind are read with one 16-byte read per lane (row l % 32, k offset 16 (l / 32) of
 // a 32-byte chunk); a K x N operand goes through the transposing reads ds_read_b64_tr_b16 /
 // _tr_b8 (within 16 lanes, lane i supplies the address of 8 bytes of k row i / 4 -- i / 2 for
-// bytes -- and receives the k-values of column i).  The row pitches spread the rows that one
+// bytes -- and receives the k-values of column i; fp32: four single-float reads, one per k row).
+// The row pitches spread the rows that one
 // read instruction touches over all banks.  Outputs leave through the element-wise epilogues of
 // the scalar any-shape kernel, so every output type and scale mode is served and nothing is
 // assumed about the alignment of C either.
