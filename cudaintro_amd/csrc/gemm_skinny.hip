@@ -245,6 +245,44 @@ __device__ __forceinline__ void sum_partials(const uint64_t* first, int64_t spli
   }
 }
 
+// The same for a number of K ranges known only at run time (up to 16): batches of up to 32 quads
+// whose loads are issued back to back under uniform conditions.
+template <typename T, int NQ>
+__device__ __forceinline__ void sum_partials_n(const uint64_t* first, int64_t split_stride,
+                                               int splits, T (&sum)[NQ][4]) {
+  constexpr int CH = 32 / NQ > 0 ? 32 / NQ : 1;  // splits per batch
+#pragma unroll
+  for (int q = 0; q < NQ; ++q)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum[q][e] = 0;
+#pragma unroll
+  for (int s0 = 0; s0 < 16; s0 += CH) {
+    if (s0 >= splits) break;
+    uint64_t lo[CH][NQ], hi[CH][NQ];
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+      if (s0 + c < splits) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+          const uint64_t* src = first + (s0 + c) * split_stride + q * 512;
+          lo[c][q] = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          hi[c][q] = __hip_atomic_load(src + 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+      if (s0 + c < splits) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+          sum[q][0] += __builtin_bit_cast(T, (uint32_t)lo[c][q]);
+          sum[q][1] += __builtin_bit_cast(T, (uint32_t)(lo[c][q] >> 32));
+          sum[q][2] += __builtin_bit_cast(T, (uint32_t)hi[c][q]);
+          sum[q][3] += __builtin_bit_cast(T, (uint32_t)(hi[c][q] >> 32));
+        }
+      }
+  }
+}
+
 // Workspace: the partials (see store_partial) followed by one arrival counter per slab.
 template <typename Geo, typename Epi, int SPLITS>
 __global__ __launch_bounds__(256, 1) void skinny_kernel(int M, int N, int stages_per_split,
@@ -608,7 +646,7 @@ struct KN16KW {
 
 template <typename Math, typename Epi, int XR, int COLS>
 __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
-    int M, int N, int stages_per_split, int splits, const char* __restrict__ X, int64_t ldx,
+    int M, int N, int stages, int splits, const char* __restrict__ X, int64_t ldx,
     const char* __restrict__ W, int64_t ldw, Epi epi, uint64_t* __restrict__ partials,
     uint32_t* __restrict__ counters, uint64_t* __restrict__ swap_words) {
   typedef KN16KW<Math::ELEM_BYTES, XR, COLS> G;
@@ -627,9 +665,11 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   const int w = __builtin_amdgcn_readfirstlane(t >> 6);
   const int slab = blockIdx.x / splits, split = blockIdx.x % splits;
   const int64_t n0 = (int64_t)slab * G::BN;
-  // this wave's k rows of the first stage of the range
-  const int64_t k0 = (int64_t)split * stages_per_split * G::K_STAGE + G::KW * w;
-  const int KTS = stages_per_split;
+  // K range `split` of `splits`: stages [split * stages / splits, (split + 1) * stages / splits),
+  // as even as the stage count allows; this wave's k rows of its first stage
+  const int s_begin = (int)((int64_t)split * stages / splits);
+  const int KTS = (int)((int64_t)(split + 1) * stages / splits) - s_begin;
+  const int64_t k0 = (int64_t)s_begin * G::K_STAGE + G::KW * w;
   char* const wave_lds = lds + w * G::WAVE_BYTES;
   const uint32_t wave_base =
       (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds + w * G::WAVE_BYTES;
@@ -800,28 +840,31 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
   if (m < M) {
     scalar_t q4[QUADS][4];
     const int64_t stride = (int64_t)slabs * G::PART_WORDS * 256;
-    switch (splits) {
-      case 2: sum_partials<scalar_t, QUADS, 2>(part(0), stride, q4); break;
-      case 4: sum_partials<scalar_t, QUADS, 4>(part(0), stride, q4); break;
-      case 8: sum_partials<scalar_t, QUADS, 8>(part(0), stride, q4); break;
-      default: sum_partials<scalar_t, QUADS, 16>(part(0), stride, q4); break;
-    }
+    sum_partials_n<scalar_t, QUADS>(part(0), stride, splits, q4);
 #pragma unroll
     for (int h = 0; h < QUADS; ++h) epi(m, n0 + c + 4 * h, q4[h][0], q4[h][1], q4[h][2], q4[h][3]);
   }
   if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// K ranges for the kernel above: a power of two, enough workgroups to cover the chip about once,
-// at least 8 stages per range, partials and counters within the workspace.
+// K ranges for the kernel above, up to 16, each of at least 8 stages, partials and counters within
+// the workspace.  One workgroup per compute unit is resident, so the count that fills the chip
+// once, floor(units / slabs), is taken when it fills at least four fifths of it (N = 5120: 80
+// slabs x 3 ranges = 240 workgroups, where a power of two gives 320 and a second round of 64:
+// 21.1 -> 16 us at K = 5120); otherwise the smallest power of two that covers the chip (N = 11008:
+// 172 slabs x 2; the second, partly filled round streams faster per unit than a full one).
 inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, int cols) {
   const int64_t slabs = N / cols;
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  if ((size_t)slabs * 4 > ctx->ws_counter_bytes) return 1;
+  auto fits = [&](int s) {
+    return s >= 1 && s <= 16 && (s == 1 || kts / s >= 8) &&
+           (s == 1 || (size_t)s * slabs * 128 * cols <= ctx->ws_partial_bytes);
+  };
+  const int fill = (int)(cus / slabs < 16 ? cus / slabs : 16);
+  if (fill >= 1 && fits(fill) && slabs * fill * 5 >= (int64_t)cus * 4) return fill;
   int s = 1;
-  while (s < 16 && slabs * s < cus && kts % (2 * s) == 0 && kts / (2 * s) >= 8 &&
-         (size_t)(2 * s) * slabs * 128 * cols <= ctx->ws_partial_bytes)
-    s *= 2;
-  if ((size_t)slabs * 4 > ctx->ws_counter_bytes) s = 1;
+  while (s < 16 && slabs * s < cus && fits(2 * s)) s *= 2;
   return s;
 }
 
@@ -836,7 +879,7 @@ void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, 
   const int64_t kts = K / G::K_STAGE;
   const int splits = kn16_kwaves_splits(ctx, N, kts, COLS);
   hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN * splits)), dim3(256), G::LDS_BYTES,
-                     ctx->stream, (int)M, (int)N, (int)(kts / splits), splits,
+                     ctx->stream, (int)M, (int)N, (int)kts, splits,
                      static_cast<const char*>(X), ldx_bytes, static_cast<const char*>(W),
                      ldw_bytes, epi, static_cast<uint64_t*>(ctx->workspace),
                      reinterpret_cast<uint32_t*>(static_cast<char*>(ctx->workspace) +
