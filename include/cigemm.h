@@ -79,8 +79,8 @@ CIGEMM_API cigemmStatus_t cigemmDestroy(cigemmHandle_t handle);
 
 /* Replaces cublasSetStream (implicit default stream in the reference).  `stream` is a
  * hipStream_t passed as void*; NULL selects the null stream.
- * The handle owns ONE workspace (64 MiB of split-K partial sums plus arrival counters,
- * allocated by cigemmCreate) that every split-K call on it uses.  Calls on one handle must
+ * The handle owns ONE workspace (64 MiB of split-K partial sums, arrival counters and 8 MiB of
+ * exchange words, allocated by cigemmCreate) that every split-K call on it uses.  Calls on one handle must
  * therefore not overlap on the device: switching the handle to another stream while work
  * enqueued on the old one may still be running, or replaying a captured graph concurrently
  * with eager calls on the same handle, races on that workspace and gives wrong results
