@@ -259,6 +259,43 @@ def k_sweep(torch, ci, wl, handle, steps, warmup):
     print(json.dumps({"k_sweep": res, "occupancy_sweep": occ}), flush=True)
 
 
+def decode_sweep(torch, ci, handle, steps, warmup):
+    """Decode GEMMs (M = 1 and 16) at layer shapes of common decoder models, bf16 K x N and int8
+    N x K weights: microseconds per call and weight bytes per second.  Several weight buffers
+    are rotated so that the Infinity Cache cannot serve them."""
+    shapes = [(4096, 4096), (11008, 4096), (4096, 11008), (12288, 4096), (5120, 5120), (13824, 5120),
+              (5120, 13824), (8192, 8192), (28672, 8192), (8192, 28672), (32000, 4096)]
+    res = {}
+    for (N, K) in shapes:
+        for M in (1, 16):
+            for kind in ("bf16", "int8"):
+                eb = 2 if kind == "bf16" else 1
+                nb = max(2, int(700e6 // (N * K * eb)) + 1)
+                if kind == "bf16":
+                    x = torch.randn((M, K), device="cuda").to(torch.bfloat16)
+                    ws = [(torch.randn((K, N), device="cuda") * 0.02).to(torch.bfloat16) for _ in range(nb)]
+                    y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+                else:
+                    x = torch.randint(-127, 128, (M, K), dtype=torch.int8, device="cuda")
+                    ws = [torch.randint(-127, 128, (N, K), dtype=torch.int8, device="cuda") for _ in range(nb)]
+                    y = torch.empty((M, N), dtype=torch.int32, device="cuda")
+                it = [0]
+
+                def fn():
+                    if kind == "bf16":
+                        handle.gemm_bf16(x, ws[it[0] % nb], out=y)
+                    else:
+                        handle.gemm_i8_i32(x, ws[it[0] % nb], ci.B_NK, out=y)
+                    it[0] += 1
+                w, e = time_calls(torch, fn, steps, warmup)
+                name = f"{kind}_M{M}_N{N}_K{K}"
+                res[name] = {"us": e / steps * 1e6, "weight_gbs": N * K * eb * steps / e / 1e9,
+                             "kernel": handle.last_kernel}
+                log(f"[decode-sweep] {name}: {json.dumps(res[name])}")
+                del ws
+    print(json.dumps({"decode_sweep": res}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -279,6 +316,9 @@ def main():
     ap.add_argument("--k-sweep", action="store_true",
                     help="instead of the benchmark: time the tile kernel at several K per M x N and "
                          "fit its fixed cost per tile and its cost per stage")
+    ap.add_argument("--decode-sweep", action="store_true",
+                    help="instead of the benchmark: decode GEMMs (M = 1, 16) at layer shapes of common "
+                         "decoder models, bf16 and int8")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1",
@@ -295,6 +335,9 @@ def main():
     handle = ci.Handle()
     if args.k_sweep:
         k_sweep(torch, ci, wl, handle, args.steps, args.warmup)
+        return
+    if args.decode_sweep:
+        decode_sweep(torch, ci, handle, args.steps, args.warmup)
         return
     n = args.size
     per_config = {}

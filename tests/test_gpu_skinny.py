@@ -191,6 +191,10 @@ def test_skinny_workspace_reuse_with_alternating_inputs(handle, torch_gpu, oracl
     (4, 1024, 4096 + 32, "32x256_ring8"),                                     # K not in whole 64-row stages
     (3, 320, 192, "32x64_kwaves"), (20, 8192 + 64, 128, "32x64_kwaves"),     # N in whole lines, not in 256s
     (32, 16384 + 192, 64, "32x64_kwaves"),
+    # three K ranges per slab (80 or 70 slabs fill the chip three times over), uneven when the
+    # stage count does not divide: 80 stages -> 26 + 27 + 27, 25 stages -> 8 + 8 + 9
+    (3, 5120, 5120, "32x64_kwaves"), (16, 5120, 13824, "32x64_kwaves"), (5, 4480, 1600, "32x64_kwaves"),
+    (8, 13824, 5120, "32x64_kwaves"),                                          # 216 slabs, one range
 ])
 def test_skinny_16bit_both_kernels_exact_inputs(handle, torch_gpu, oracle, rng, kind, M, N, K, kernel):
     """The two 16-bit decode kernels (64-column slabs with K over the waves; 256-column slabs with
