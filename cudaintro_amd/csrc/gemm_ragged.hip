@@ -102,11 +102,55 @@ __device__ __forceinline__ u32x4 fetch_piece_narrow(const T* __restrict__ P, int
   return v;
 }
 
+// Split-K: the accumulators of one K range, stored raw (fp32 or int32 bits) to
+// base[split * split_stride + r * ld + c]; a second kernel sums the ranges in order and applies
+// the real epilogue, one element per lane.
+struct EpiPartialElem {
+  uint32_t* base;
+  int64_t ld;
+  int64_t split_stride;
+  template <typename T>
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, T acc) const {
+    base[r * ld + c] = __builtin_bit_cast(uint32_t, acc);
+  }
+};
+template <typename Epi>
+__device__ __forceinline__ Epi any_epilogue_of_split(const Epi& e, int) { return e; }
+__device__ __forceinline__ EpiPartialElem any_epilogue_of_split(const EpiPartialElem& e, int split) {
+  return EpiPartialElem{e.base + split * e.split_stride, e.ld, e.split_stride};
+}
+
+template <typename Scalar, typename Epi>
+__global__ __launch_bounds__(256) void any_reduce_kernel(int64_t M, int64_t N, int splits,
+                                                         const uint32_t* __restrict__ part,
+                                                         int64_t split_stride, Epi epi) {
+  const int64_t total = M * N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * 256) {
+    // all ranges are read before the first add waits for one (splits <= 16)
+    uint32_t v[16];
+#pragma unroll
+    for (int sp = 0; sp < 16; ++sp)
+      if (sp < splits) v[sp] = part[sp * split_stride + i];
+    Scalar sum = __builtin_bit_cast(Scalar, v[0]);
+#pragma unroll
+    for (int sp = 1; sp < 16; ++sp)
+      if (sp < splits) sum += __builtin_bit_cast(Scalar, v[sp]);
+    epi(i / N, i % N, sum);
+  }
+}
+
 template <typename Math, bool B_NK, typename Epi>
 __global__ __launch_bounds__(256) void mfma_any_kernel(int64_t M, int64_t N, int64_t K,
                                                        const void* __restrict__ Av, int64_t lda,
                                                        const void* __restrict__ Bv, int64_t ldb,
-                                                       Epi epi, int tiles_m, int tiles_n) {
+                                                       Epi epi_all, int tiles_m, int tiles_n,
+                                                       int64_t k_range) {
+  // blockIdx.y = K range (split launches only): k in [y * k_range, min(K, (y + 1) * k_range)),
+  // k_range a multiple of the step; the rest of the kernel sees that range as its K
+  const Epi epi = any_epilogue_of_split(epi_all, (int)blockIdx.y);
+  const int64_t k_begin = (int64_t)blockIdx.y * k_range;
+  K = K < k_begin + k_range ? K : k_begin + k_range;
   typedef RaggedElem<Math::ELEM_BYTES> E;
   typedef typename E::type elem_t;
   typedef typename Math::acc_t acc_t;
@@ -230,8 +274,8 @@ __global__ __launch_bounds__(256) void mfma_any_kernel(int64_t M, int64_t N, int
   };
 
   auto run = [&](auto narrow) {
-    fetch(0, narrow);
-    for (int64_t k0 = 0; k0 < K; k0 += KE) {
+    fetch(k_begin, narrow);
+    for (int64_t k0 = k_begin; k0 < K; k0 += KE) {
       stash(k0, narrow);
       __syncthreads();
       if (k0 + KE < K) fetch(k0 + KE, narrow);  // in flight while this step multiplies
@@ -285,33 +329,72 @@ __global__ __launch_bounds__(256) void mfma_any_kernel(int64_t M, int64_t N, int
     }
 }
 
+// K ranges for a problem of few tiles (a decode or small-batch shape that no aligned kernel
+// takes): about three workgroups per compute unit are resident, so enough ranges to fill those
+// places, each of at least four steps, at most 16, partials within the workspace.  N = 8191,
+// K = 8192, M = 1 (64 tiles): 255 us unsplit.
+template <typename Math>
+int any_splits(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K, int64_t tiles) {
+  constexpr int KE = RK / Math::ELEM_BYTES;
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  if (!ctx->workspace || tiles * 2 > 3 * (int64_t)cus) return 1;  // fewer than two ranges fit
+  const int64_t steps = (K + KE - 1) / KE;
+  int64_t s = 3 * (int64_t)cus / tiles;
+  if (s > 16) s = 16;
+  if (s > steps / 4) s = steps / 4;
+  while (s > 1 && (size_t)s * (size_t)M * (size_t)N * 4 > ctx->ws_partial_bytes) --s;
+  return s < 1 ? 1 : (int)s;
+}
+
+// Returns the number of K ranges the problem was run in.
 template <typename Math, bool B_NK, typename Epi>
-void launch_any(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
-                const void* B, int64_t ldb, const Epi& epi) {
+int launch_any(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+               const void* B, int64_t ldb, const Epi& epi) {
+  typedef typename Math::scalar_t scalar_t;
+  constexpr int KE = RK / Math::ELEM_BYTES;
   const int tiles_m = (int)((M + RT - 1) / RT), tiles_n = (int)((N + RT - 1) / RT);
-  hipLaunchKernelGGL((mfma_any_kernel<Math, B_NK, Epi>), dim3((unsigned)(tiles_m * tiles_n)),
-                     dim3(256), 0, ctx->stream, M, N, K, A, lda, B, ldb, epi, tiles_m, tiles_n);
+  const int64_t tiles = (int64_t)tiles_m * tiles_n;
+  int splits = any_splits<Math>(ctx, M, N, K, tiles);
+  // steps per range, rounded up; ranges that would start past K are dropped
+  const int64_t steps = (K + KE - 1) / KE;
+  const int64_t k_range = splits > 1 ? (steps + splits - 1) / splits * KE : (K > 0 ? K : 1);
+  if (splits > 1) splits = (int)((K + k_range - 1) / k_range);
+  if (splits <= 1) {
+    hipLaunchKernelGGL((mfma_any_kernel<Math, B_NK, Epi>), dim3((unsigned)tiles), dim3(256), 0,
+                       ctx->stream, M, N, K, A, lda, B, ldb, epi, tiles_m, tiles_n, k_range);
+    return 1;
+  }
+  uint32_t* ws = static_cast<uint32_t*>(ctx->workspace);
+  hipLaunchKernelGGL((mfma_any_kernel<Math, B_NK, EpiPartialElem>),
+                     dim3((unsigned)tiles, (unsigned)splits), dim3(256), 0, ctx->stream, M, N, K, A,
+                     lda, B, ldb, EpiPartialElem{ws, N, M * N}, tiles_m, tiles_n, k_range);
+  const int64_t blocks = (M * N + 255) / 256;
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  hipLaunchKernelGGL((any_reduce_kernel<scalar_t, Epi>),
+                     dim3((unsigned)(blocks < 8 * (int64_t)cus ? blocks : 8 * (int64_t)cus)),
+                     dim3(256), 0, ctx->stream, M, N, splits, ws, M * N, epi);
+  return splits;
+}
+
+// "<name>" or "<name>_splitk", kept in the context
+void set_any_name(cigemmContext* ctx, const char* name, int splits) {
+  snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s%s", name, splits > 1 ? "_splitk" : "");
+  ctx->last_kernel = ctx->kernel_name;
 }
 
 template <bool B_NK>
-void launch_any_i8_layout(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
-                          int64_t lda, const int8_t* B, int64_t ldb, int32_t* C, int64_t ldc,
-                          const DequantArgs* dq) {
-  if (!dq) {
-    launch_any<tile::MathI8, B_NK>(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32{C, ldc});
-    return;
-  }
+int launch_any_i8_layout(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
+                         int64_t lda, const int8_t* B, int64_t ldb, int32_t* C, int64_t ldc,
+                         const DequantArgs* dq) {
+  if (!dq) return launch_any<tile::MathI8, B_NK>(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32{C, ldc});
   const bool dump = dq->acc_out != nullptr;
 #define CIG_DQ(OB, DA)                                                                        \
   launch_any<tile::MathI8, B_NK>(ctx, M, N, K, A, lda, B, ldb,                                 \
                                  EpiDequant<OB, DA>{dq->out, dq->ldo, dq->sa, dq->sb,          \
                                                     dq->sa_vec, dq->sb_vec, dq->acc_out,       \
                                                     dq->ldacc})
-  if (dq->out_bf16) {
-    if (dump) CIG_DQ(true, true); else CIG_DQ(true, false);
-  } else {
-    if (dump) CIG_DQ(false, true); else CIG_DQ(false, false);
-  }
+  if (dq->out_bf16) return dump ? CIG_DQ(true, true) : CIG_DQ(true, false);
+  return dump ? CIG_DQ(false, true) : CIG_DQ(false, false);
 #undef CIG_DQ
 }
 
@@ -327,13 +410,14 @@ bool launch_mfma_any_16(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int
                         const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                         uint16_t* C, int64_t ldc) {
   if (!any_shape_ok(M, N)) return false;
-  if (bf16) {
-    launch_any<tile::MathBF16, false>(ctx, M, N, K, A, lda, B, ldb, EpiStore16<BF16>{C, ldc});
-    ctx->last_kernel = "bf16_mfma_any_128x128x32";
-  } else {
-    launch_any<tile::MathF16, false>(ctx, M, N, K, A, lda, B, ldb, EpiStore16<F16>{C, ldc});
-    ctx->last_kernel = "f16_mfma_any_128x128x32";
-  }
+  if (bf16)
+    set_any_name(ctx, "bf16_mfma_any_128x128x32",
+                 launch_any<tile::MathBF16, false>(ctx, M, N, K, A, lda, B, ldb,
+                                                   EpiStore16<BF16>{C, ldc}));
+  else
+    set_any_name(ctx, "f16_mfma_any_128x128x32",
+                 launch_any<tile::MathF16, false>(ctx, M, N, K, A, lda, B, ldb,
+                                                  EpiStore16<F16>{C, ldc}));
   return true;
 }
 
@@ -341,14 +425,14 @@ bool launch_mfma_any_f32(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, co
                          int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
                          const BiasAct* ba) {
   if (!any_shape_ok(M, N)) return false;
-  if (ba) {
-    launch_any<tile::MathF32, false>(ctx, M, N, K, A, lda, B, ldb,
-                                     EpiBiasActF32{C, ldc, ba->bias, ba->relu});
-    ctx->last_kernel = "f32_mfma_any_128x128x16_bias_act";
-  } else {
-    launch_any<tile::MathF32, false>(ctx, M, N, K, A, lda, B, ldb, EpiStoreF32{C, ldc});
-    ctx->last_kernel = "f32_mfma_any_128x128x16";
-  }
+  if (ba)
+    set_any_name(ctx, "f32_mfma_any_128x128x16_bias_act",
+                 launch_any<tile::MathF32, false>(ctx, M, N, K, A, lda, B, ldb,
+                                                  EpiBiasActF32{C, ldc, ba->bias, ba->relu}));
+  else
+    set_any_name(ctx, "f32_mfma_any_128x128x16",
+                 launch_any<tile::MathF32, false>(ctx, M, N, K, A, lda, B, ldb,
+                                                  EpiStoreF32{C, ldc}));
   return true;
 }
 
@@ -356,12 +440,12 @@ bool launch_mfma_any_i8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, con
                         int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
                         int64_t ldc, const DequantArgs* dq) {
   if (!any_shape_ok(M, N)) return false;
-  if (b_nk)
-    launch_any_i8_layout<true>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
-  else
-    launch_any_i8_layout<false>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
-  ctx->last_kernel = b_nk ? (dq ? "i8_mfma_any_128x128x64_nk_dequant" : "i8_mfma_any_128x128x64_nk")
-                          : (dq ? "i8_mfma_any_128x128x64_kn_dequant" : "i8_mfma_any_128x128x64_kn");
+  const int splits = b_nk ? launch_any_i8_layout<true>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq)
+                          : launch_any_i8_layout<false>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
+  set_any_name(ctx,
+               b_nk ? (dq ? "i8_mfma_any_128x128x64_nk_dequant" : "i8_mfma_any_128x128x64_nk")
+                    : (dq ? "i8_mfma_any_128x128x64_kn_dequant" : "i8_mfma_any_128x128x64_kn"),
+               splits);
   return true;
 }
 

@@ -13,7 +13,10 @@ pytestmark = pytest.mark.gpu
 
 VALS = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
 SHAPES = [(1, 1, 1), (3, 5, 7), (64, 63, 64), (129, 131, 67), (300, 257, 1000), (128, 128, 33),
-          (17, 1000, 129), (260, 4, 2049)]
+          (17, 1000, 129), (260, 4, 2049),
+          # few tiles and a long K: run as K ranges into the workspace plus a reduction launch
+          (1, 2047, 2050), (16, 1000, 4097), (130, 257, 3001)]
+SPLIT = {(1, 2047, 2050), (16, 1000, 4097), (130, 257, 3001), (260, 4, 2049), (300, 257, 1000)}
 
 
 def embed(torch, a, dtype, off, pad, fill):
@@ -52,6 +55,7 @@ def test_any_shape_16bit(handle, torch_gpu, oracle, rng, kind, M, N, K):
             with handle.algo(algo):
                 fn(a, b, out=out)
             assert "mfma_any" in handle.last_kernel, handle.last_kernel
+            assert handle.last_kernel.endswith("_splitk") == ((M, N, K) in SPLIT), handle.last_kernel
             got = bits(torch, out)
             if exact:
                 np.testing.assert_array_equal(got, narrow(oracle.gemm_f32(widen(Ab), widen(Bb))))
