@@ -608,20 +608,20 @@ bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, cons
   return false;
 }
 
-// ---- 16-bit, K x N weights, 64-column slabs: K over the waves, at most a two-way exchange ---
-// The kernel above gives a workgroup 256 columns and splits K over up to 16 workgroups per slab,
-// so its reduction reads up to 16 partial tiles per slab.  Here a workgroup owns 64 columns --
-// one whole 128-byte line of every weight row, the narrowest slab whose requests are not half
-// lines -- and a K range; inside it the four waves split k (a stage is 64 rows of k, wave w moves
-// and multiplies rows 16 w .. 16 w + 15 of every stage and never touches what another wave
-// moved: no workgroup barrier in the loop), their four partial 32 x 64 tiles are summed through
-// LDS in wave order, and only then do K ranges meet, through the same partial / arrival-counter
-// exchange as above.  N = 8192 gives 128 slabs, so two K ranges fill 256 compute units: the
-// last workgroup of a slab reads one partial tile instead of seven.
-// Per wave and stage: the W piece [16 k][64 n] (2 KiB, two DMA instructions of 8 whole lines) and
-// the x piece [XR m][16 k] (XR x 32 bytes of the slot, XR = 8, 16 or 32, the smallest that holds
-// M; one DMA instruction of 2 M lanes fills its first M rows), in a ring of NSTAGES slots private
-// to the wave.
+// ---- K x N weights, slabs of whole lines: K over the waves ------------------------------------
+// The kernel above gives a workgroup 256 columns and a workgroup barrier per stage, and splits K
+// over up to 16 workgroups per slab.  Here a workgroup owns a slab of one or two whole 128-byte
+// lines of every weight row (64 or 128 columns of a 16-bit type, 128 of int8; half lines stream
+// at two thirds of the rate) and a K range; inside it the four waves split k (a stage is 64 rows
+// of k -- 128 for int8 --, wave w moves and multiplies rows 16 w .. 16 w + 15 of every stage and
+// never touches what another wave moved: no workgroup barrier in the loop), their four partial
+// 32-row tiles are summed through LDS in wave order, and only then do K ranges meet: two ranges
+// through one atomic exchange per pair of outputs, more through the partial / arrival-counter
+// exchange of the kernel above.
+// Per wave and stage: the W piece [16 k][slab] (2 or 4 KiB, DMA instructions of 1 KiB of whole
+// rows each) and the x piece [XR m][16 k] (XR x 32 bytes of the slot, XR = 8, 16 or 32, the
+// smallest that holds M; one DMA instruction of 2 M lanes fills its first M rows), in a ring of
+// NSTAGES slots private to the wave.
 template <int EB_, int XR_, int COLS_>
 struct KN16KW {
   static constexpr int EB = EB_;                       // bytes per element: 2 (fp16, bf16) or 1 (int8)
@@ -635,7 +635,7 @@ struct KN16KW {
   static constexpr int W_DMAS = W_BYTES / 1024;        // one instruction moves 1 KiB of whole rows
   static constexpr int X_BYTES = XR * 32;              // 32 bytes of k per row of x
   static constexpr int SLOT_BYTES = W_BYTES + X_BYTES;
-  static constexpr int NSTAGES = W_BYTES == 1024 ? 16 : W_BYTES == 2048 ? 12 : 7;
+  static constexpr int NSTAGES = W_BYTES == 1024 ? 16 : W_BYTES == 2048 ? 12 : W_BYTES == 4096 ? 7 : 4;
   static constexpr int DPS = W_DMAS + 1;               // DMA instructions per wave and stage
   static constexpr int WAVE_BYTES = NSTAGES * SLOT_BYTES;
   static constexpr int RED_LD = BN + 4;                // words per row of the reduction tiles
@@ -892,12 +892,11 @@ void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, 
                          : nullptr);
 }
 
-// COLS = 64, one line per weight row, is the only width in use.  Two lines per row (128-column
-// slabs: half the x traffic per weight byte, half as many slabs) was measured for 17 to 32 rows
-// of x: 1 % faster than the 256-column kernel at N = K = 8192, 2-5 % at N = 16384, much slower
-// than 64 columns below.  Half a line per row (32-column slabs: 256 slabs at N = 8192, no
+// Slab widths of the 16-bit types: 64 columns (one line per weight row) and 128 (two lines);
+// kn16_choice says which.  Half a line per row (32-column slabs: 256 slabs at N = 8192, no
 // exchange between workgroups at all) streams at two thirds of the rate: 45 against 30 us at
-// N = K = 8192, 47 against 28 at 16384 x 4096, level only at N = 1024.
+// N = K = 8192, 47 against 28 at 16384 x 4096, level only at N = 1024.  int8 K x N weights use
+// 128 columns (one line); 256 columns were measured slower there (8192 x 8192: 17.8 -> 19.2 us).
 template <typename Math, int COLS, typename Epi>
 void launch_kn16_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
                         int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
@@ -932,11 +931,18 @@ struct Slab32 {
 // 31.2 -> 30.5 at M = 16) except with more than 16 rows of x over many slabs (M = 32 at N = K =
 // 8192: 32.7 against 34.1 us; at N = K = 4096 still 20.3 -> 12.7).
 // A shape that only one of the two takes (N a multiple of 64 but not of 256; K a multiple of 32
-// but not of 64) goes to that one.  0: neither, 1: 64-column slabs, 2: 256-column slabs.
+// but not of 64) goes to that one.  Large weight matrices take the K-over-the-waves kernel with
+// 128-column slabs -- two lines, 256 contiguous bytes, per weight row and DMA row -- which
+// streams faster and re-reads x half as often (N = K = 8192: 29.5 -> 26.8 us at M = 1, 32.4 ->
+// 29.5 at M = 32; 28672 x 8192: 95.7 -> 80.3 us; 6144 x 6144: 24.4 -> 17.6), at the price of
+// half as many slabs, so twice the K ranges to exchange: slower below 32 slabs or 2048 k
+// (2048 x 8192: 12.1 -> 13.1 us, 8192 x 1024: 7.1 -> 7.9).
+// 0: neither, 1: 64-column slabs, 2: 256-column slabs with a barrier per stage, 3: 128-column slabs.
 inline int kn16_choice(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K) {
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
   const bool kw_ok = N % 64 == 0 && K % 64 == 0 && (size_t)(N / 64) * 4 <= ctx->ws_counter_bytes;
   const bool sk_ok = N % GeoKN16<tile::MathBF16>::BN == 0 && K % GeoKN16<tile::MathBF16>::K_ELEMS == 0;
+  if (kw_ok && N % 128 == 0 && N / 128 >= 32 && K >= 2048) return 3;
   if (kw_ok && (M <= 16 || N / 64 < cus / 2 || !sk_ok)) return 1;
   return sk_ok ? 2 : 0;
 }
@@ -950,6 +956,10 @@ const char* launch_skinny_16_on(cigemmContext* ctx, int64_t M, int64_t N, int64_
                                 const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                                 uint16_t* C, int64_t ldc, bool bf16) {
   const int which = kn16_choice(ctx, M, N, K);
+  if (which == 3) {
+    launch_kn16_kwaves<Math, 128>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
+    return bf16 ? "bf16_skinny_32x128_kwaves" : "f16_skinny_32x128_kwaves";
+  }
   if (which == 1) {
     launch_kn16_kwaves<Math, 64>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
     return bf16 ? "bf16_skinny_32x64_kwaves" : "f16_skinny_32x64_kwaves";

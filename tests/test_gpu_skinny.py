@@ -184,17 +184,19 @@ def test_skinny_workspace_reuse_with_alternating_inputs(handle, torch_gpu, oracl
 
 @pytest.mark.parametrize("kind", ["bf16", "f16"])
 @pytest.mark.parametrize("M,N,K,kernel", [
-    (1, 256, 64, "32x64_kwaves"), (3, 512, 1024, "32x64_kwaves"), (8, 8192, 8192, "32x64_kwaves"),
-    (16, 8192, 4096, "32x64_kwaves"), (17, 4096, 4096, "32x64_kwaves"), (32, 2048, 8192, "32x64_kwaves"),
-    (32, 256, 3072, "32x64_kwaves"), (5, 16384, 2048, "32x64_kwaves"),
-    (17, 8192, 1024, "32x256_ring8"), (32, 8192, 8192, "32x256_ring8"),     # many rows of x over many slabs
+    (1, 256, 64, "32x64_kwaves"), (3, 512, 1024, "32x64_kwaves"), (32, 2048, 8192, "32x64_kwaves"),
+    (32, 256, 3072, "32x64_kwaves"), (16, 8192, 1024, "32x64_kwaves"),
+    # large weight matrices (at least 32 slabs of 128 columns, 2048 k): 128-column slabs
+    (8, 8192, 8192, "32x128_kwaves"), (16, 8192, 4096, "32x128_kwaves"), (17, 4096, 4096, "32x128_kwaves"),
+    (5, 16384, 2048, "32x128_kwaves"), (32, 8192, 8192, "32x128_kwaves"),
+    (17, 8192, 1024, "32x256_ring8"),                                         # many rows of x, short K
     (4, 1024, 4096 + 32, "32x256_ring8"),                                     # K not in whole 64-row stages
     (3, 320, 192, "32x64_kwaves"), (20, 8192 + 64, 128, "32x64_kwaves"),     # N in whole lines, not in 256s
-    (32, 16384 + 192, 64, "32x64_kwaves"),
-    # three K ranges per slab (80 or 70 slabs fill the chip three times over), uneven when the
-    # stage count does not divide: 80 stages -> 26 + 27 + 27, 25 stages -> 8 + 8 + 9
-    (3, 5120, 5120, "32x64_kwaves"), (16, 5120, 13824, "32x64_kwaves"), (5, 4480, 1600, "32x64_kwaves"),
-    (8, 13824, 5120, "32x64_kwaves"),                                          # 216 slabs, one range
+    (32, 16384 + 192, 64, "32x64_kwaves"), (9, 8192 + 64, 4096, "32x64_kwaves"),
+    # K ranges that fill the chip once, uneven when the stage count does not divide: 40 slabs x 6
+    # ranges of 80 stages (13 or 14 each), 70 slabs x 3 of 25 stages (8 + 8 + 9), 108 slabs x 2
+    (3, 5120, 5120, "32x128_kwaves"), (16, 5120, 13824, "32x128_kwaves"), (5, 4480, 1600, "32x64_kwaves"),
+    (8, 13824, 5120, "32x128_kwaves"),
 ])
 def test_skinny_16bit_both_kernels_exact_inputs(handle, torch_gpu, oracle, rng, kind, M, N, K, kernel):
     """The two 16-bit decode kernels (64-column slabs with K over the waves; 256-column slabs with
@@ -217,15 +219,17 @@ def test_skinny_16bit_both_kernels_exact_inputs(handle, torch_gpu, oracle, rng, 
         assert (got[M:] == narrow(np.float32(7.0))).all()
 
 
+@pytest.mark.parametrize("N,K,kernel", [(16384, 4096, "32x128"), (8192 + 64, 4096, "32x64")])
 @pytest.mark.parametrize("zero_part", ["all", "first_range", "second_range", "columns"])
-def test_two_range_exchange_with_zero_partial_sums(handle, torch_gpu, oracle, rng, zero_part):
-    """N = 8192 gives the 64-column kernel two K ranges per slab, which meet through one atomic
-    exchange per pair of outputs; a pair of +0.0 partial sums looks like the exchange word's empty
-    state and travels as -0.0.  Weights that are zero over a whole K range, over everything, or
-    in some columns give such pairs; the results must equal the CPU loop's bits (+0.0 where the
-    sum is zero), three calls in a row (every word returns to empty)."""
+def test_two_range_exchange_with_zero_partial_sums(handle, torch_gpu, oracle, rng, zero_part, N, K, kernel):
+    """128 slabs (16384 columns in 128-column slabs, 8256 in 64-column ones) get two K ranges
+    each, which meet through one atomic exchange per pair of outputs; a pair of +0.0 partial sums
+    looks like the exchange word's empty state and travels as -0.0.  Weights that are zero over a
+    whole K range, over everything, or in some columns give such pairs; the results must equal
+    the CPU loop's bits (+0.0 where the sum is zero), three calls in a row (every word returns to
+    empty)."""
     torch = torch_gpu
-    M, N, K = 3, 8192, 8192
+    M = 3
     vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
     X, W = rng.choice(vals, size=(M, K)), rng.choice(vals, size=(K, N))
     W[rng.random(size=W.shape) < 0.5] = 0
@@ -242,7 +246,7 @@ def test_two_range_exchange_with_zero_partial_sums(handle, torch_gpu, oracle, rn
     x, w = to_dev(torch, oracle.f32_to_bf16(X), "bf16"), to_dev(torch, oracle.f32_to_bf16(W), "bf16")
     for _ in range(3):
         y = handle.gemm_bf16(x, w)
-        assert handle.last_kernel == "bf16_skinny_32x64_kwaves", handle.last_kernel
+        assert handle.last_kernel == f"bf16_skinny_{kernel}_kwaves", handle.last_kernel
         np.testing.assert_array_equal(bits(torch, y), want)
 
 
