@@ -585,6 +585,11 @@ void launch_skinny_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, c
                      static_cast<const char*>(W), ldw_bytes, epi);
 }
 
+// (A variant with 1024-byte stages, each wave moving 256 contiguous bytes of every weight row --
+// 4 rows x 256 bytes per DMA instruction, as the 16-bit kernel's 128-column slabs do -- was built
+// and measured for M <= 8: slower, 17.8 against 14.1 us at N = K = 8192, with its ring of four
+// 40 KiB stages; level only at K = 28672.  Not kept.)
+//
 // int8 N x K: the kernel above unless the weights are a few slabs of a very long K (then the
 // K ranges of the split-K kernel spread the stream over more compute units).  Measured at
 // M = 8, per call: 4096 x 8192 13.2 -> 10.1 us, 4096 x 4096 10.9 -> 7.2, 1024 x 8192 11.1 ->
