@@ -630,8 +630,8 @@ bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, cons
 template <int EB_, int XR_, int COLS_>
 struct KN16KW {
   static constexpr int EB = EB_;                       // bytes per element: 2 (fp16, bf16) or 1 (int8)
-  static constexpr int BN = COLS_;                     // 16-bit: 64 (one line per weight row; 32 and
-                                                       // 128 were measured); int8: 128 (one line)
+  static constexpr int BN = COLS_;                     // 16-bit: 64 or 128 (one or two lines per
+                                                       // weight row); int8: 128 (one line)
   static constexpr int KW = 32 / EB;                   // k rows per wave and stage = one MFMA's k
   static constexpr int K_STAGE = 4 * KW;               // k rows per stage and workgroup
   static constexpr int XR = XR_;
@@ -854,10 +854,11 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
 
 // K ranges for the kernel above, up to 16, each of at least 8 stages, partials and counters within
 // the workspace.  One workgroup per compute unit is resident, so the count that fills the chip
-// once, floor(units / slabs), is taken when it fills at least four fifths of it (N = 5120: 80
-// slabs x 3 ranges = 240 workgroups, where a power of two gives 320 and a second round of 64:
-// 21.1 -> 16 us at K = 5120); otherwise the smallest power of two that covers the chip (N = 11008:
-// 172 slabs x 2; the second, partly filled round streams faster per unit than a full one).
+// once, floor(units / slabs), is taken when it fills at least four fifths of it (N = 5120 in
+// 64-column slabs: 80 slabs x 3 ranges = 240 workgroups, where a power of two gives 320 and a
+// second round of 64: 21.1 -> 16 us at K = 5120); otherwise the smallest power of two that covers
+// the chip (N = 11008: 86 slabs of 128 columns x 4; the second, partly filled round streams
+// faster per unit than a full one).
 inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, int cols) {
   const int64_t slabs = N / cols;
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
