@@ -20,6 +20,9 @@
 //
 // int8 weights with at least one 32-column slab per compute unit take a second kernel that
 // needs none of that: K is split over the four waves of the workgroup (further down).
+// K x N weights (16-bit, int8) with N and K multiples of 64 (int8: 128) take a third one: slabs
+// of one or two whole 128-byte lines per weight row, K over the waves, short rings so that two
+// workgroups fit a compute unit (further down; it serves nearly every 16-bit decode shape).
 #include <atomic>
 #include <cstdarg>
 #include <mutex>
@@ -450,7 +453,7 @@ void launch_skinny(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const vo
 // summed through LDS in wave order at the end.  No partials in memory, no arrival counter, no
 // second pass: the three dependent trips through the fabric that the split-K fix-up costs
 // (about 5 us per call) are gone.
-template <int XR_>
+template <int XR_, bool DEEP_ = false>
 struct NK8KW {
   static constexpr int BN = 32;
   static constexpr int K_ELEMS = 512;
@@ -458,18 +461,23 @@ struct NK8KW {
   static constexpr int W_BYTES = 32 * 512;           // four [32 n][128 B] sub-tiles, one per wave
   static constexpr int X_BYTES = XR * 512;           // four [XR m][128 B] sub-tiles
   static constexpr int STAGE_BYTES = W_BYTES + X_BYTES;
-  static constexpr int NSTAGES = XR == 8 ? 7 : XR == 16 ? 6 : 5;   // 140 / 144 / 160 KiB
+  // Two workgroups share the LDS of a compute unit (60 / 72 / 64 KiB each): with more slabs
+  // than units nobody waits for a second round, and with fewer the shallower ring is no slower
+  // (M = 8: N = K = 8192 13.9 -> 13.1 us, 11008 x 4096 15.1 -> 12.7, 28672 x 8192 47.8 ->
+  // 43.1) -- except with 32 rows of x, where a ring of two stages is: then the deep ring
+  // (160 KiB, one workgroup per unit) while the slabs fit one round.
+  static constexpr int NSTAGES = DEEP_ ? 5 : XR == 32 ? 2 : 3;
   static constexpr int DPS = 4 + XR / 8;             // per wave and stage, 1 KiB each
 };
 
-template <typename Epi, int XR>
-__global__ __launch_bounds__(256, 1) void skinny_nk8_kwaves_kernel(int M, int N, int K,
+template <typename Epi, int XR, bool DEEP>
+__global__ __launch_bounds__(256, 2) void skinny_nk8_kwaves_kernel(int M, int N, int K,
                                                                    const char* __restrict__ X,
                                                                    int64_t ldx,
                                                                    const char* __restrict__ W,
                                                                    int64_t ldw, Epi epi) {
   typedef tile::MathI8 Math;
-  typedef NK8KW<XR> G;
+  typedef NK8KW<XR, DEEP> G;
   constexpr int NS = G::NSTAGES, DIST = NS - 1;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int t = threadIdx.x, l = t & 63;
@@ -571,18 +579,32 @@ __global__ __launch_bounds__(256, 1) void skinny_nk8_kwaves_kernel(int M, int N,
   epi(m, n0 + c, sum[0], sum[1], sum[2], sum[3]);
 }
 
-template <typename Epi, int XR>
-void launch_skinny_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
-                          int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
-  typedef NK8KW<XR> G;
+template <typename Epi, int XR, bool DEEP>
+void launch_skinny_kwaves_ring(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
+                               int64_t ldx_bytes, const void* W, int64_t ldw_bytes,
+                               const Epi& epi) {
+  typedef NK8KW<XR, DEEP> G;
   constexpr int LDS_BYTES = G::NSTAGES * G::STAGE_BYTES;
-  static_assert(LDS_BYTES <= 160 * 1024, "ring must fit the LDS");
-  auto kern = skinny_nk8_kwaves_kernel<Epi, XR>;
+  static_assert(LDS_BYTES * (DEEP ? 1 : 2) <= 160 * 1024, "rings must fit the LDS");
+  auto kern = skinny_nk8_kwaves_kernel<Epi, XR, DEEP>;
   static std::atomic<uint64_t> lds_set{0};
   if (!ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set)) return;
   hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN)), dim3(256), LDS_BYTES, ctx->stream, (int)M,
                      (int)N, (int)K, static_cast<const char*>(X), ldx_bytes,
                      static_cast<const char*>(W), ldw_bytes, epi);
+}
+
+template <typename Epi, int XR>
+void launch_skinny_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
+                          int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
+  if constexpr (XR == 32) {
+    const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+    if (N / NK8KW<XR>::BN <= cus) {
+      launch_skinny_kwaves_ring<Epi, XR, true>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+      return;
+    }
+  }
+  launch_skinny_kwaves_ring<Epi, XR, false>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
 }
 
 // (A variant with 1024-byte stages, each wave moving 256 contiguous bytes of every weight row --
@@ -626,7 +648,12 @@ bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, cons
 // Per wave and stage: the W piece [16 k][slab] (2 or 4 KiB, DMA instructions of 1 KiB of whole
 // rows each) and the x piece [XR m][16 k] (XR x 32 bytes of the slot, XR = 8, 16 or 32, the
 // smallest that holds M; one DMA instruction of 2 M lanes fills its first M rows), in a ring of
-// NSTAGES slots private to the wave.
+// NSTAGES slots private to the wave.  The rings are short enough for two workgroups to share a
+// compute unit's LDS (3 or 4 slots beside 4 KiB W pieces, 6 beside 2 KiB): a launch of more
+// workgroups than units then has no second round that waits for the first, and a single
+// workgroup on a unit streams no slower than with rings twice as deep (measured, M = 1 / 32, 7
+// slots -> 4 / 3: N = K = 8192 26.6 / 29.5 -> 26.1 / 28.4 us, 28672 x 8192 80.4 / 90.7 ->
+// 79.8 / 85.1).
 template <int EB_, int XR_, int COLS_>
 struct KN16KW {
   static constexpr int EB = EB_;                       // bytes per element: 2 (fp16, bf16) or 1 (int8)
@@ -640,7 +667,8 @@ struct KN16KW {
   static constexpr int W_DMAS = W_BYTES / 1024;        // one instruction moves 1 KiB of whole rows
   static constexpr int X_BYTES = XR * 32;              // 32 bytes of k per row of x
   static constexpr int SLOT_BYTES = W_BYTES + X_BYTES;
-  static constexpr int NSTAGES = W_BYTES == 1024 ? 16 : W_BYTES == 2048 ? 12 : W_BYTES == 4096 ? 7 : 4;
+  // ring slots per wave: what lets two workgroups share the LDS of a compute unit
+  static constexpr int NSTAGES = W_BYTES <= 1024 ? 8 : W_BYTES == 2048 ? 6 : XR <= 16 ? 4 : 3;
   static constexpr int DPS = W_DMAS + 1;               // DMA instructions per wave and stage
   static constexpr int WAVE_BYTES = NSTAGES * SLOT_BYTES;
   static constexpr int RED_LD = BN + 4;                // words per row of the reduction tiles
@@ -650,7 +678,7 @@ struct KN16KW {
 };
 
 template <typename Math, typename Epi, int XR, int COLS>
-__global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
+__global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
     int M, int N, int stages, int splits, const char* __restrict__ X, int64_t ldx,
     const char* __restrict__ W, int64_t ldw, Epi epi, uint64_t* __restrict__ partials,
     uint32_t* __restrict__ counters, uint64_t* __restrict__ swap_words) {
@@ -853,32 +881,36 @@ __global__ __launch_bounds__(256, 1) void skinny_kn16_kwaves_kernel(
 }
 
 // K ranges for the kernel above, up to 16, each of at least 8 stages, partials and counters within
-// the workspace.  One workgroup per compute unit is resident, so the count that fills the chip
-// once, floor(units / slabs), is taken when it fills at least four fifths of it (N = 5120 in
-// 64-column slabs: 80 slabs x 3 ranges = 240 workgroups, where a power of two gives 320 and a
-// second round of 64: 21.1 -> 16 us at K = 5120); otherwise the smallest power of two that covers
-// the chip (N = 11008: 86 slabs of 128 columns x 4; the second, partly filled round streams
-// faster per unit than a full one).
+// the workspace.  Two workgroups fit a compute unit, and the ones that share a unit share its
+// rate: a launch takes about (stages per range) x (workgroups on the fullest unit), so that is
+// what the count minimises, the fewest ranges on a tie.  N = K = 8192 in 128-column slabs: 64
+// slabs x 4 ranges = one workgroup per unit.  N = 11008, K = 4096: 86 slabs x 5 = 430
+// workgroups, two on most units (20.4 us; 4 ranges, two on a third of the units, 22.3; 2
+// ranges, 172 units busy, 20.9; 3 ranges 23.8).  N = 13824, K = 5120: 108 slabs x 2.
 inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, int cols) {
   const int64_t slabs = N / cols;
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
   if ((size_t)slabs * 4 > ctx->ws_counter_bytes) return 1;
-  auto fits = [&](int s) {
-    return s >= 1 && s <= 16 && (s == 1 || kts / s >= 8) &&
-           (s == 1 || (size_t)s * slabs * 128 * cols <= ctx->ws_partial_bytes);
-  };
-  const int fill = (int)(cus / slabs < 16 ? cus / slabs : 16);
-  if (fill >= 1 && fits(fill) && slabs * fill * 5 >= (int64_t)cus * 4) return fill;
-  int s = 1;
-  while (s < 16 && slabs * s < cus && fits(2 * s)) s *= 2;
-  return s;
+  int best = 1;
+  int64_t best_cost = kts * ((slabs + cus - 1) / cus) * 16;  // in sixteenths of a stage
+  for (int s = 2; s <= 16; ++s) {
+    if (kts / s < 8 || slabs * s > 2 * cus) break;
+    if ((size_t)s * slabs * 128 * cols > ctx->ws_partial_bytes) break;
+    const int64_t cost = (kts * 16 / s) * ((slabs * s + cus - 1) / cus);
+    if (cost * 10 < best_cost * 9) {  // more ranges must pay for their exchange
+      best_cost = cost;
+      best = s;
+    }
+  }
+  return best;
 }
 
 template <typename Math, typename Epi, int XR, int COLS>
 void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const void* X,
                            int64_t ldx_bytes, const void* W, int64_t ldw_bytes, const Epi& epi) {
   typedef KN16KW<Math::ELEM_BYTES, XR, COLS> G;
-  static_assert(G::LDS_BYTES + 64 <= 160 * 1024, "rings and the arrival flag must fit the LDS");
+  static_assert(2 * (G::LDS_BYTES + 64) <= 160 * 1024,
+                "rings and arrival flags of two workgroups must fit the LDS");
   auto kern = skinny_kn16_kwaves_kernel<Math, Epi, XR, COLS>;
   static std::atomic<uint64_t> lds_set{0};
   if (!ensure_dynamic_lds(ctx, (const void*)kern, G::LDS_BYTES, lds_set)) return;
@@ -931,25 +963,26 @@ struct Slab32 {
   static constexpr int BN = 32, K_ELEMS = 128;
 };
 
-// Which 16-bit decode kernel.  The 64-column one needs whole stages of 64 k per range and pays
-// for its narrow slabs with four times the x traffic of the 256-column one: faster everywhere
-// (N = K = 4096: 19.4 -> 11.2 us, 2048 x 8192: 19.4 -> 11.5, N = K = 8192: 30.9 -> 30.0 at M = 1,
-// 31.2 -> 30.5 at M = 16) except with more than 16 rows of x over many slabs (M = 32 at N = K =
-// 8192: 32.7 against 34.1 us; at N = K = 4096 still 20.3 -> 12.7).
-// A shape that only one of the two takes (N a multiple of 64 but not of 256; K a multiple of 32
-// but not of 64) goes to that one.  Large weight matrices take the K-over-the-waves kernel with
-// 128-column slabs -- two lines, 256 contiguous bytes, per weight row and DMA row -- which
-// streams faster and re-reads x half as often (N = K = 8192: 29.5 -> 26.8 us at M = 1, 32.4 ->
-// 29.5 at M = 32; 28672 x 8192: 95.7 -> 80.3 us; 6144 x 6144: 24.4 -> 17.6), at the price of
-// half as many slabs, so twice the K ranges to exchange: slower below 32 slabs or 2048 k
-// (2048 x 8192: 12.1 -> 13.1 us, 8192 x 1024: 7.1 -> 7.9).
+// Which 16-bit decode kernel.  The K-over-the-waves kernel takes every shape it can (N and K
+// multiples of 64); the 256-column kernel with a barrier per stage is left with K a multiple of
+// 32 but not of 64 (with N a multiple of 256), where it is the only one: everywhere else it is
+// slower, up to twice with more than 16 rows of x (N = 8192, K = 1024, M = 32: 14.1 against
+// 7.2 us; N = K = 4096: 19.4 against 10.7 at M = 1).
+// Slab width: large weight matrices take 128-column slabs -- two lines, 256 contiguous bytes,
+// per weight row and DMA row -- which stream faster and re-read x half as often (M = 1 / 32:
+// N = K = 8192 28.4 / 32.0 -> 26.0 / 28.4 us, 28672 x 8192 95.9 / 127.4 -> 79.4 / 84.6, 22016 x
+// 4096 44.3 / 59.1 -> 34.1 / 38.9, 6144 x 6144 18.0 / 22.4 -> 17.3 / 19.2), at the price of half
+// as many slabs, so twice the K ranges to exchange: no faster up to 4096 x 4096 weights (level
+// there and at 8192 x 2048; 4096 x 2048: 7.8 / 8.5 against 8.0 / 9.6), slower below 32 slabs or
+// 2048 k (2048 x 8192: 11.1 / 12.4 against 13.0 / 15.8 us, 8192 x 1024: 7.1 / 7.3 against 7.4 /
+// 8.8).
 // 0: neither, 1: 64-column slabs, 2: 256-column slabs with a barrier per stage, 3: 128-column slabs.
-inline int kn16_choice(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K) {
-  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+inline int kn16_choice(const cigemmContext* ctx, int64_t N, int64_t K) {
   const bool kw_ok = N % 64 == 0 && K % 64 == 0 && (size_t)(N / 64) * 4 <= ctx->ws_counter_bytes;
   const bool sk_ok = N % GeoKN16<tile::MathBF16>::BN == 0 && K % GeoKN16<tile::MathBF16>::K_ELEMS == 0;
-  if (kw_ok && N % 128 == 0 && N / 128 >= 32 && K >= 2048) return 3;
-  if (kw_ok && (M <= 16 || N / 64 < cus / 2 || !sk_ok)) return 1;
+  if (kw_ok && N % 128 == 0 && N / 128 >= 32 && K >= 2048 && N * K > (int64_t)4096 * 4096)
+    return 3;
+  if (kw_ok) return 1;
   return sk_ok ? 2 : 0;
 }
 
@@ -961,7 +994,7 @@ template <typename Math, typename E16>
 const char* launch_skinny_16_on(cigemmContext* ctx, int64_t M, int64_t N, int64_t K,
                                 const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                                 uint16_t* C, int64_t ldc, bool bf16) {
-  const int which = kn16_choice(ctx, M, N, K);
+  const int which = kn16_choice(ctx, N, K);
   if (which == 3) {
     launch_kn16_kwaves<Math, 128>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
     return bf16 ? "bf16_skinny_32x128_kwaves" : "f16_skinny_32x128_kwaves";

@@ -98,7 +98,8 @@ def test_skinny_int8_nk(handle, torch_gpu, oracle, rng, M, N, K, out_type):
 @pytest.mark.parametrize("M", [1, 5, 8, 9, 16, 17, 32])
 @pytest.mark.parametrize("N,K", [(8192, 512), (8192 + 128, 1536), (8192, 4096 + 128), (128, 128), (256, 640),
                                  (32, 256), (8192 + 96, 1024), (160, 16384 + 640),
-                                 (2048, 16384 + 384), (256, 16384 + 512), (1024, 32768 + 128)])
+                                 (2048, 16384 + 384), (256, 16384 + 512), (1024, 32768 + 128),
+                                 (11008, 1024)])
 def test_skinny_int8_without_split_k(handle, torch_gpu, oracle, rng, M, N, K):
     """The kernel that splits K over the waves of a workgroup instead of over workgroups, with
     8, 16 or 32 rows of x per stage and a last stage of one to four k-chunks.  A few slabs of
@@ -186,10 +187,11 @@ def test_skinny_workspace_reuse_with_alternating_inputs(handle, torch_gpu, oracl
 @pytest.mark.parametrize("M,N,K,kernel", [
     (1, 256, 64, "32x64_kwaves"), (3, 512, 1024, "32x64_kwaves"), (32, 2048, 8192, "32x64_kwaves"),
     (32, 256, 3072, "32x64_kwaves"), (16, 8192, 1024, "32x64_kwaves"),
-    # large weight matrices (at least 32 slabs of 128 columns, 2048 k): 128-column slabs
-    (8, 8192, 8192, "32x128_kwaves"), (16, 8192, 4096, "32x128_kwaves"), (17, 4096, 4096, "32x128_kwaves"),
+    # large weight matrices (at least 32 slabs of 128 columns, 2048 k, more than 4096 x 4096
+    # weights): 128-column slabs
+    (8, 8192, 8192, "32x128_kwaves"), (16, 8192, 4096, "32x128_kwaves"), (17, 4096, 8192, "32x128_kwaves"),
     (5, 16384, 2048, "32x128_kwaves"), (32, 8192, 8192, "32x128_kwaves"),
-    (17, 8192, 1024, "32x256_ring8"),                                         # many rows of x, short K
+    (17, 4096, 4096, "32x64_kwaves"), (17, 8192, 1024, "32x64_kwaves"), (32, 8192, 2048, "32x64_kwaves"),
     (4, 1024, 4096 + 32, "32x256_ring8"),                                     # K not in whole 64-row stages
     (3, 320, 192, "32x64_kwaves"), (20, 8192 + 64, 128, "32x64_kwaves"),     # N in whole lines, not in 256s
     (32, 16384 + 192, 64, "32x64_kwaves"), (9, 8192 + 64, 4096, "32x64_kwaves"),
@@ -197,6 +199,10 @@ def test_skinny_workspace_reuse_with_alternating_inputs(handle, torch_gpu, oracl
     # ranges of 80 stages (13 or 14 each), 70 slabs x 3 of 25 stages (8 + 8 + 9), 108 slabs x 2
     (3, 5120, 5120, "32x128_kwaves"), (16, 5120, 13824, "32x128_kwaves"), (5, 4480, 1600, "32x64_kwaves"),
     (8, 13824, 5120, "32x128_kwaves"),
+    # more workgroups than compute units, two to a unit: 86 slabs x 5 ranges of 64 stages (12 or 13
+    # each), 96 x 5, 129 slabs of 64 columns x 3; 172 slabs in one range each
+    (8, 11008, 4096, "32x128_kwaves"), (32, 12288, 4096, "32x128_kwaves"), (20, 8192 + 64, 4096, "32x64_kwaves"),
+    (2, 22016, 4096, "32x128_kwaves"),
 ])
 def test_skinny_16bit_both_kernels_exact_inputs(handle, torch_gpu, oracle, rng, kind, M, N, K, kernel):
     """The two 16-bit decode kernels (64-column slabs with K over the waves; 256-column slabs with
@@ -219,11 +225,11 @@ def test_skinny_16bit_both_kernels_exact_inputs(handle, torch_gpu, oracle, rng, 
         assert (got[M:] == narrow(np.float32(7.0))).all()
 
 
-@pytest.mark.parametrize("N,K,kernel", [(16384, 4096, "32x128"), (8192 + 64, 4096, "32x64")])
+@pytest.mark.parametrize("N,K,kernel", [(16384, 4096, "32x128"), (8192 - 64, 1024, "32x64")])
 @pytest.mark.parametrize("zero_part", ["all", "first_range", "second_range", "columns"])
 def test_two_range_exchange_with_zero_partial_sums(handle, torch_gpu, oracle, rng, zero_part, N, K, kernel):
-    """128 slabs (16384 columns in 128-column slabs, 8256 in 64-column ones) get two K ranges
-    each, which meet through one atomic exchange per pair of outputs; a pair of +0.0 partial sums
+    """128 slabs of 128 columns over 64 stages, or 127 slabs of 64 columns over 16 stages, get two
+    K ranges each, which meet through one atomic exchange per pair of outputs; a pair of +0.0 partial sums
     looks like the exchange word's empty state and travels as -0.0.  Weights that are zero over a
     whole K range, over everything, or in some columns give such pairs; the results must equal
     the CPU loop's bits (+0.0 where the sum is zero), three calls in a row (every word returns to
