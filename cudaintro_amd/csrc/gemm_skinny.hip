@@ -464,8 +464,10 @@ struct NK8KW {
   // Two workgroups share the LDS of a compute unit (60 / 72 / 64 KiB each): with more slabs
   // than units nobody waits for a second round, and with fewer the shallower ring is no slower
   // (M = 8: N = K = 8192 13.9 -> 13.1 us, 11008 x 4096 15.1 -> 12.7, 28672 x 8192 47.8 ->
-  // 43.1) -- except with 32 rows of x, where a ring of two stages is: then the deep ring
-  // (160 KiB, one workgroup per unit) while the slabs fit one round.
+  // 43.1).  With 32 rows of x only two stages fit beside a second workgroup, and that ring is
+  // slower when a workgroup has its unit to itself (N = K = 8192: 14.8 -> 16.4 us), faster with
+  // more slabs than units (16384 x 4096: 19.9 -> 15.2): DEEP_ is the ring of 5 stages (160 KiB,
+  // one workgroup per unit) for the first case.
   static constexpr int NSTAGES = DEEP_ ? 5 : XR == 32 ? 2 : 3;
   static constexpr int DPS = 4 + XR / 8;             // per wave and stage, 1 KiB each
 };
@@ -883,7 +885,8 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
 // K ranges for the kernel above, up to 16, each of at least 8 stages, partials and counters within
 // the workspace.  Two workgroups fit a compute unit, and the ones that share a unit share its
 // rate: a launch takes about (stages per range) x (workgroups on the fullest unit), so that is
-// what the count minimises, the fewest ranges on a tie.  N = K = 8192 in 128-column slabs: 64
+// what the count minimises; more ranges are taken only when they make it a tenth smaller (their
+// exchange costs, too).  N = K = 8192 in 128-column slabs: 64
 // slabs x 4 ranges = one workgroup per unit.  N = 11008, K = 4096: 86 slabs x 5 = 430
 // workgroups, two on most units (20.4 us; 4 ranges, two on a third of the units, 22.3; 2
 // ranges, 172 units busy, 20.9; 3 ranges 23.8).  N = 13824, K = 5120: 108 slabs x 2.
