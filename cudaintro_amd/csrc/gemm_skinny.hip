@@ -29,6 +29,7 @@
 
 #include "epilogues.h"
 #include "mfma_tile.h"
+#include "skinny_plan.h"
 
 namespace cig {
 namespace {
@@ -882,30 +883,10 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
   if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// K ranges for the kernel above, up to 16, each of at least 8 stages, partials and counters within
-// the workspace.  Two workgroups fit a compute unit, and the ones that share a unit share its
-// rate: a launch takes about (stages per range) x (workgroups on the fullest unit), so that is
-// what the count minimises; more ranges are taken only when they make it a tenth smaller (their
-// exchange costs, too).  N = K = 8192 in 128-column slabs: 64
-// slabs x 4 ranges = one workgroup per unit.  N = 11008, K = 4096: 86 slabs x 5 = 430
-// workgroups, two on most units (20.4 us; 4 ranges, two on a third of the units, 22.3; 2
-// ranges, 172 units busy, 20.9; 3 ranges 23.8).  N = 13824, K = 5120: 108 slabs x 2.
+// K ranges per slab for the kernel above: skinny_plan.h has the rule.
 inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, int cols) {
-  const int64_t slabs = N / cols;
-  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-  if ((size_t)slabs * 4 > ctx->ws_counter_bytes) return 1;
-  int best = 1;
-  int64_t best_cost = kts * ((slabs + cus - 1) / cus) * 16;  // in sixteenths of a stage
-  for (int s = 2; s <= 16; ++s) {
-    if (kts / s < 8 || slabs * s > 2 * cus) break;
-    if ((size_t)s * slabs * 128 * cols > ctx->ws_partial_bytes) break;
-    const int64_t cost = (kts * 16 / s) * ((slabs * s + cus - 1) / cus);
-    if (cost * 10 < best_cost * 9) {  // more ranges must pay for their exchange
-      best_cost = cost;
-      best = s;
-    }
-  }
-  return best;
+  return skinny_plan::kwaves_splits(N / cols, kts, cols, ctx->num_cus, ctx->ws_counter_bytes,
+                                    ctx->ws_partial_bytes);
 }
 
 template <typename Math, typename Epi, int XR, int COLS>

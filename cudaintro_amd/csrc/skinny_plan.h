@@ -1,0 +1,38 @@
+// Launch planning of the K-over-the-waves decode kernel (gemm_skinny.hip), as plain host
+// functions of sizes so that a host-only test can check them.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+
+namespace cig {
+namespace skinny_plan {
+
+// K ranges per slab, up to 16, each of at least 8 stages, partials (128 bytes per column, slab
+// and range: 32 rows of 4-byte sums) and counters (4 bytes per slab) within the workspace.  Two
+// workgroups fit a compute unit, and the ones that share a unit share its rate: a launch takes
+// about (stages per range) x (workgroups on the fullest unit), so that is what the count
+// minimises; more ranges are taken only when they make it a tenth smaller (their exchange
+// costs, too).  N = K = 8192 in 128-column slabs: 64 slabs x 4 ranges = one workgroup per unit.
+// N = 11008, K = 4096: 86 slabs x 5 = 430 workgroups, two on most units (20.4 us; 4 ranges, two
+// on a third of the units, 22.3; 2 ranges, 172 units busy, 20.9; 3 ranges 23.8).  N = 13824,
+// K = 5120: 108 slabs x 2.
+inline int kwaves_splits(int64_t slabs, int64_t stages, int cols, int cus, size_t counter_bytes,
+                         size_t partial_bytes) {
+  if (cus <= 0) cus = 256;
+  if ((size_t)slabs * 4 > counter_bytes) return 1;
+  int best = 1;
+  int64_t best_cost = stages * ((slabs + cus - 1) / cus) * 16;  // in sixteenths of a stage
+  for (int s = 2; s <= 16; ++s) {
+    if (stages / s < 8 || slabs * s > 2 * (int64_t)cus) break;
+    if ((size_t)s * (size_t)slabs * 128 * (size_t)cols > partial_bytes) break;
+    const int64_t cost = (stages * 16 / s) * ((slabs * s + cus - 1) / cus);
+    if (cost * 10 < best_cost * 9) {
+      best_cost = cost;
+      best = s;
+    }
+  }
+  return best;
+}
+
+}  // namespace skinny_plan
+}  // namespace cig

@@ -1,0 +1,69 @@
+// Host-only checks of the decode kernel's launch planning (csrc/skinny_plan.h): invariants over a
+// sweep of sizes, and the counts the measurements behind the rule were taken at.
+#include <cstdio>
+#include <cstdlib>
+#include <initializer_list>
+
+#include "skinny_plan.h"
+
+using cig::skinny_plan::kwaves_splits;
+
+static int failures = 0;
+#define EXPECT(cond)                                                     \
+  do {                                                                   \
+    if (!(cond)) {                                                       \
+      std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);      \
+      ++failures;                                                        \
+    }                                                                    \
+  } while (0)
+
+int main() {
+  const size_t counters = 4096, partials = (size_t)64 << 20;
+  // 16-bit weights: a stage is 64 k
+  EXPECT(kwaves_splits(8192 / 128, 8192 / 64, 128, 256, counters, partials) == 4);
+  EXPECT(kwaves_splits(11008 / 128, 4096 / 64, 128, 256, counters, partials) == 5);
+  EXPECT(kwaves_splits(12288 / 128, 4096 / 64, 128, 256, counters, partials) == 5);
+  EXPECT(kwaves_splits(13824 / 128, 5120 / 64, 128, 256, counters, partials) == 2);
+  EXPECT(kwaves_splits(22016 / 128, 4096 / 64, 128, 256, counters, partials) == 1);
+  EXPECT(kwaves_splits(28672 / 128, 8192 / 64, 128, 256, counters, partials) == 1);
+  EXPECT(kwaves_splits(6144 / 128, 6144 / 64, 128, 256, counters, partials) == 5);
+  EXPECT(kwaves_splits(5120 / 128, 5120 / 64, 128, 256, counters, partials) == 6);
+  EXPECT(kwaves_splits(16384 / 128, 4096 / 64, 128, 256, counters, partials) == 2);
+  EXPECT(kwaves_splits(4096 / 64, 4096 / 64, 64, 256, counters, partials) == 4);
+  EXPECT(kwaves_splits(1024 / 64, 8192 / 64, 64, 256, counters, partials) == 16);
+  EXPECT(kwaves_splits(8128 / 64, 1024 / 64, 64, 256, counters, partials) == 2);
+  EXPECT(kwaves_splits(4480 / 64, 1600 / 64, 64, 256, counters, partials) == 3);
+  // int8 K x N weights: a stage is 128 k
+  EXPECT(kwaves_splits(11008 / 128, 4096 / 128, 128, 256, counters, partials) == 2);
+  EXPECT(kwaves_splits(8192 / 128, 8192 / 128, 128, 256, counters, partials) == 4);
+  // no room for counters or partials: no exchange
+  EXPECT(kwaves_splits(2000, 512, 64, 256, counters, partials) == 1);
+  EXPECT(kwaves_splits(64, 128, 128, 256, counters, 0) == 1);
+  EXPECT(kwaves_splits(64, 128, 128, 256, counters, (size_t)3 * 64 * 128 * 128) == 3);
+  // a device that does not report its units counts as 256
+  EXPECT(kwaves_splits(64, 128, 128, 0, counters, partials) == 4);
+
+  // invariants over a sweep
+  long checked = 0;
+  for (int cus : {32, 64, 120, 256, 304})
+    for (int cols : {64, 128})
+      for (int64_t slabs = 1; slabs <= 1200; slabs += (slabs < 300 ? 1 : 37))
+        for (int64_t stages = 1; stages <= 600; stages += (stages < 40 ? 1 : 13)) {
+          const int s = kwaves_splits(slabs, stages, cols, cus, counters, partials);
+          ++checked;
+          EXPECT(s >= 1 && s <= 16);
+          if (s > 1) {
+            EXPECT(stages / s >= 8);                 // ranges of at least 8 stages
+            EXPECT(slabs * s <= 2 * (int64_t)cus);   // at most two workgroups per unit
+            EXPECT((size_t)slabs * 4 <= counters);
+            EXPECT((size_t)s * slabs * 128 * cols <= partials);
+            // never worse than a single range by the rule's own measure
+            EXPECT((stages * 16 / s) * ((slabs * s + cus - 1) / cus) <
+                   stages * 16 * ((slabs + cus - 1) / cus));
+          }
+          if (failures > 20) return 1;
+        }
+  if (failures) return 1;
+  std::printf("skinny plan OK (%ld cases)\n", checked);
+  return 0;
+}

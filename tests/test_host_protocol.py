@@ -17,6 +17,17 @@ def test_host_protocol(tmp_path):
     assert "host protocol OK" in out.stdout
 
 
+def test_skinny_plan(tmp_path):
+    """The decode kernel's choice of K ranges (csrc/skinny_plan.h): the counts the rule was
+    measured at, and its invariants over a sweep of sizes."""
+    exe = tmp_path / "test_skinny_plan"
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(ROOT, "cudaintro_amd", "csrc"),
+                    os.path.join(ROOT, "tests", "cpp", "test_skinny_plan.cpp"), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "skinny plan OK" in out.stdout
+
+
 def test_gemm_common_header_names():
     """The drop-in header keeps the record and the four entry-point names."""
     text = open(os.path.join(ROOT, "include", "gemm_common.h")).read()
