@@ -668,16 +668,18 @@ struct KN16KW {
   static constexpr int ROW_BYTES = EB * BN;
   static constexpr int W_BYTES = KW * ROW_BYTES;       // per wave and stage
   static constexpr int W_DMAS = W_BYTES / 1024;        // one instruction moves 1 KiB of whole rows
+  static constexpr int MT = XR > 32 ? 2 : 1;           // 32-row tiles of x (XR = 64: two)
   static constexpr int X_BYTES = XR * 32;              // 32 bytes of k per row of x
   static constexpr int SLOT_BYTES = W_BYTES + X_BYTES;
   // ring slots per wave: what lets two workgroups share the LDS of a compute unit
   static constexpr int NSTAGES = W_BYTES <= 1024 ? 8 : W_BYTES == 2048 ? 6 : XR <= 16 ? 4 : 3;
-  static constexpr int DPS = W_DMAS + 1;               // DMA instructions per wave and stage
+  static constexpr int DPS = W_DMAS + MT;              // DMA instructions per wave and stage
   static constexpr int WAVE_BYTES = NSTAGES * SLOT_BYTES;
   static constexpr int RED_LD = BN + 4;                // words per row of the reduction tiles
   static constexpr int RED_BYTES = 4 * 32 * RED_LD * 4;
   static constexpr int LDS_BYTES = 4 * WAVE_BYTES > RED_BYTES ? 4 * WAVE_BYTES : RED_BYTES;
-  static constexpr int PART_WORDS = BN / 16;           // 64-bit words per thread of a partial tile
+  static constexpr int PART_WORDS = BN / 16;           // 64-bit words per thread and 32-row tile
+                                                       // of a partial result
 };
 
 template <typename Math, typename Epi, int XR, int COLS>
@@ -692,6 +694,7 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
   constexpr int EB = G::EB;
   constexpr int NS = G::NSTAGES, DIST = NS - 1;
   constexpr int NT = COLS / 32;                       // 32-column tiles of the slab
+  constexpr int MT = G::MT;                           // 32-row tiles of x
   constexpr int PIECES = G::ROW_BYTES / 16;           // 16-byte pieces of a slab row
   constexpr int ROWS_PER_DMA = 64 / PIECES;
   constexpr int QUADS = COLS / 32;                    // groups of 4 columns per thread of the reduction
@@ -722,13 +725,19 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
 #pragma unroll
     for (int i = 0; i < G::W_DMAS; ++i) dma16(ws + (int64_t)(ROWS_PER_DMA * i) * ldw, dst + 1024 * i);
     if (l < 2 * M) dma16(x_src + st * (G::K_STAGE * EB), dst + G::W_BYTES);
+    // rows 32 and up (the launcher picks XR = 64 only for M > 32: lane 0 always takes part, so
+    // the instruction is issued and counted every time)
+    if constexpr (MT == 2)
+      if (l + 64 < 2 * M) dma16(x_src + 32 * ldx + st * (G::K_STAGE * EB), dst + G::W_BYTES + 1024);
   };
 
-  typename Math::acc_t acc[NT];
+  typename Math::acc_t acc[MT][NT];
 #pragma unroll
-  for (int j = 0; j < NT; ++j)
+  for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[j][e] = 0;
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 #pragma unroll
   for (int st = 0; st < DIST; ++st)
     if (st < KTS) issue(st, st);
@@ -742,7 +751,7 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
                                   (16 * ((l >> 4) & 1) + 4 * (l & 3)) * 2
                             : (16 * (l >> 5) + ((l & 15) >> 1)) * G::ROW_BYTES +
                                   16 * ((l >> 4) & 1) + 8 * (l & 1);
-  const int x_off = G::W_BYTES + (l & (XR - 1)) * 32 + ((l >> 5) << 4);
+  const int x_off = G::W_BYTES + (l & ((XR < 32 ? XR : 32) - 1)) * 32 + ((l >> 5) << 4);
   int slot = 0, dma_slot = DIST;
   for (int s = 0; s < KTS; ++s) {
     // Stage s landed for this wave; nothing is fetched past the K range, so fewer stages are
@@ -752,7 +761,9 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
     __builtin_amdgcn_sched_barrier(0);
     if (s + DIST < KTS) issue(s + DIST, dma_slot);
     const char* sl = wave_lds + slot * G::SLOT_BYTES;
-    const u32x4 xf = *reinterpret_cast<const u32x4*>(sl + x_off);
+    u32x4 xf[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xf[i] = *reinterpret_cast<const u32x4*>(sl + x_off + 1024 * i);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       u32x4 wf;
@@ -769,49 +780,60 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
         wf = __builtin_shufflevector(__builtin_bit_cast(u32x2, lo), __builtin_bit_cast(u32x2, hi),
                                      0, 1, 2, 3);
       }
-      acc[j] = Math::mfma(wf, xf, acc[j]);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) acc[i][j] = Math::mfma(wf, xf[i], acc[i][j]);
     }
     slot = slot + 1 == NS ? 0 : slot + 1;
     dma_slot = dma_slot + 1 == NS ? 0 : dma_slot + 1;
   }
   __syncthreads();  // every wave done with its ring (nothing is in flight): reuse it
 
-  // acc[j][4 q + e] = this wave's part of y[l % 32][n0 + 32 j + 8 q + 4 (l / 32) + e]
+  // acc[i][j][4 q + e] = this wave's part of y[32 i + l % 32][n0 + 32 j + 8 q + 4 (l / 32) + e].
+  // One 32-row tile of x at a time goes through the reduction tiles: thread t takes row t / 8
+  // (+ 32 i), columns 4 QUADS (t % 8) .. + 4 QUADS - 1, summed over the waves in wave order.
   scalar_t* red = reinterpret_cast<scalar_t*>(lds);  // [4 waves][32 m][RED_LD]
+  const int m0 = t >> 3, c = (t & 7) * 4 * QUADS;
+  scalar_t sums[MT][4 * QUADS];
 #pragma unroll
-  for (int j = 0; j < NT; ++j)
+  for (int i = 0; i < MT; ++i) {
+    if (i > 0) __syncthreads();  // the tiles of the rows before are read
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      scalar_t* dst = red + (w * 32 + (l & 31)) * G::RED_LD + 32 * j + 8 * q + 4 * (l >> 5);
-      const u32x4 v = {__builtin_bit_cast(uint32_t, (scalar_t)acc[j][4 * q]),
-                       __builtin_bit_cast(uint32_t, (scalar_t)acc[j][4 * q + 1]),
-                       __builtin_bit_cast(uint32_t, (scalar_t)acc[j][4 * q + 2]),
-                       __builtin_bit_cast(uint32_t, (scalar_t)acc[j][4 * q + 3])};
-      *reinterpret_cast<u32x4*>(dst) = v;
-    }
-  __syncthreads();
-  // thread t: row t / 8, columns 4 QUADS (t % 8) .. + 4 QUADS - 1, summed over the waves in
-  // wave order
-  const int m = t >> 3, c = (t & 7) * 4 * QUADS;
-  scalar_t sum[4 * QUADS];
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-  for (int h = 0; h < QUADS; ++h) {
+      for (int q = 0; q < 4; ++q) {
+        scalar_t* dst = red + (w * 32 + (l & 31)) * G::RED_LD + 32 * j + 8 * q + 4 * (l >> 5);
+        const u32x4 v = {__builtin_bit_cast(uint32_t, (scalar_t)acc[i][j][4 * q]),
+                         __builtin_bit_cast(uint32_t, (scalar_t)acc[i][j][4 * q + 1]),
+                         __builtin_bit_cast(uint32_t, (scalar_t)acc[i][j][4 * q + 2]),
+                         __builtin_bit_cast(uint32_t, (scalar_t)acc[i][j][4 * q + 3])};
+        *reinterpret_cast<u32x4*>(dst) = v;
+      }
+    __syncthreads();
 #pragma unroll
-    for (int ww = 0; ww < 4; ++ww) {
-      const u32x4 p = *reinterpret_cast<const u32x4*>(red + (ww * 32 + m) * G::RED_LD + c + 4 * h);
+    for (int h = 0; h < QUADS; ++h) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t bits = p[e];
-        const scalar_t v = __builtin_bit_cast(scalar_t, bits);
-        sum[4 * h + e] = ww == 0 ? v : sum[4 * h + e] + v;
+      for (int ww = 0; ww < 4; ++ww) {
+        const u32x4 p =
+            *reinterpret_cast<const u32x4*>(red + (ww * 32 + m0) * G::RED_LD + c + 4 * h);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t bits = p[e];
+          const scalar_t v = __builtin_bit_cast(scalar_t, bits);
+          sums[i][4 * h + e] = ww == 0 ? v : sums[i][4 * h + e] + v;
+        }
       }
     }
   }
   if (splits == 1) {
-    if (m < M) {
 #pragma unroll
-      for (int h = 0; h < QUADS; ++h)
-        epi(m, n0 + c + 4 * h, sum[4 * h], sum[4 * h + 1], sum[4 * h + 2], sum[4 * h + 3]);
+    for (int i = 0; i < MT; ++i) {
+      const int m = m0 + 32 * i;
+      if (m < M) {
+#pragma unroll
+        for (int h = 0; h < QUADS; ++h)
+          epi(m, n0 + c + 4 * h, sums[i][4 * h], sums[i][4 * h + 1], sums[i][4 * h + 2],
+              sums[i][4 * h + 3]);
+      }
     }
     return;
   }
@@ -827,43 +849,54 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
   // -0.0f, which 0 + x turns back into +0.0f.
   if constexpr (EB == 2) {
   if (splits == 2 && swap_words) {
-    if (m < M) {
-      uint64_t* word = swap_words + ((int64_t)slab * G::PART_WORDS) * 256 + t;
-      uint64_t got[2 * QUADS];
 #pragma unroll
-      for (int p = 0; p < 2 * QUADS; ++p) {
-        uint64_t mine = (uint64_t)__builtin_bit_cast(uint32_t, sum[2 * p]) |
-                        ((uint64_t)__builtin_bit_cast(uint32_t, sum[2 * p + 1]) << 32);
-        if (mine == 0) mine = 0x8000000080000000ull;
-        got[p] = __hip_atomic_exchange(word + 256 * p, mine, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-      }
+    for (int i = 0; i < MT; ++i) {
+      const int m = m0 + 32 * i;
+      const scalar_t* sum = sums[i];
+      if (m < M) {
+        uint64_t* word = swap_words + ((int64_t)(slab * MT + i) * G::PART_WORDS) * 256 + t;
+        uint64_t got[2 * QUADS];
 #pragma unroll
-      for (int p = 0; p < 2 * QUADS; ++p) {
-        if (got[p] == 0) continue;
-        const float o0 = __builtin_bit_cast(float, (uint32_t)got[p]);
-        const float o1 = __builtin_bit_cast(float, (uint32_t)(got[p] >> 32));
-        const float a0 = split == 0 ? sum[2 * p] : o0, b0 = split == 0 ? o0 : sum[2 * p];
-        const float a1 = split == 0 ? sum[2 * p + 1] : o1, b1 = split == 0 ? o1 : sum[2 * p + 1];
-        epi.pair(m, n0 + c + 2 * p, (0.0f + a0) + b0, (0.0f + a1) + b1);
-        __hip_atomic_store(word + 256 * p, (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int p = 0; p < 2 * QUADS; ++p) {
+          uint64_t mine = (uint64_t)__builtin_bit_cast(uint32_t, sum[2 * p]) |
+                          ((uint64_t)__builtin_bit_cast(uint32_t, sum[2 * p + 1]) << 32);
+          if (mine == 0) mine = 0x8000000080000000ull;
+          got[p] = __hip_atomic_exchange(word + 256 * p, mine, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int p = 0; p < 2 * QUADS; ++p) {
+          if (got[p] == 0) continue;
+          const float o0 = __builtin_bit_cast(float, (uint32_t)got[p]);
+          const float o1 = __builtin_bit_cast(float, (uint32_t)(got[p] >> 32));
+          const float a0 = split == 0 ? sum[2 * p] : o0, b0 = split == 0 ? o0 : sum[2 * p];
+          const float a1 = split == 0 ? sum[2 * p + 1] : o1,
+                      b1 = split == 0 ? o1 : sum[2 * p + 1];
+          epi.pair(m, n0 + c + 2 * p, (0.0f + a0) + b0, (0.0f + a1) + b1);
+          __hip_atomic_store(word + 256 * p, (uint64_t)0, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+        }
       }
     }
     return;
   }
   }
   // ---- more K ranges: same exchange as in skinny_kernel (partials as agent-scope 64-bit words,
-  // laid out [split][slab][word][thread]; the last workgroup of the slab sums in split order)
+  // laid out [split][slab][tile of x][word][thread]; the last workgroup of the slab sums in split
+  // order)
   const int slabs = gridDim.x / splits;
-  auto part = [&](int sp) {
-    return partials + ((int64_t)(sp * slabs + slab) * G::PART_WORDS) * 256 + t;
+  auto part = [&](int sp, int i) {
+    return partials + ((int64_t)((sp * slabs + slab) * MT + i) * G::PART_WORDS) * 256 + t;
   };
-  if (m < M) {
-    uint64_t* dst = part(split);
 #pragma unroll
-    for (int h = 0; h < QUADS; ++h)
-      store_partial(dst + 512 * h, sum[4 * h], sum[4 * h + 1], sum[4 * h + 2], sum[4 * h + 3]);
-  }
+  for (int i = 0; i < MT; ++i)
+    if (m0 + 32 * i < M) {
+      uint64_t* dst = part(split, i);
+#pragma unroll
+      for (int h = 0; h < QUADS; ++h)
+        store_partial(dst + 512 * h, sums[i][4 * h], sums[i][4 * h + 1], sums[i][4 * h + 2],
+                      sums[i][4 * h + 3]);
+    }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's partial stores are acknowledged
   __syncthreads();
   if (t == 0) {
@@ -873,20 +906,26 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
   }
   __syncthreads();
   if (!is_last) return;
-  if (m < M) {
-    scalar_t q4[QUADS][4];
-    const int64_t stride = (int64_t)slabs * G::PART_WORDS * 256;
-    sum_partials_n<scalar_t, QUADS>(part(0), stride, splits, q4);
 #pragma unroll
-    for (int h = 0; h < QUADS; ++h) epi(m, n0 + c + 4 * h, q4[h][0], q4[h][1], q4[h][2], q4[h][3]);
+  for (int i = 0; i < MT; ++i) {
+    const int m = m0 + 32 * i;
+    if (m < M) {
+      scalar_t q4[QUADS][4];
+      const int64_t stride = (int64_t)slabs * MT * G::PART_WORDS * 256;
+      sum_partials_n<scalar_t, QUADS>(part(0, i), stride, splits, q4);
+#pragma unroll
+      for (int h = 0; h < QUADS; ++h)
+        epi(m, n0 + c + 4 * h, q4[h][0], q4[h][1], q4[h][2], q4[h][3]);
+    }
   }
   if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // K ranges per slab for the kernel above: skinny_plan.h has the rule.
-inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, int cols) {
+inline int kn16_kwaves_splits(const cigemmContext* ctx, int64_t N, int64_t kts, int cols,
+                              int x_tiles) {
   return skinny_plan::kwaves_splits(N / cols, kts, cols, ctx->num_cus, ctx->ws_counter_bytes,
-                                    ctx->ws_partial_bytes);
+                                    ctx->ws_partial_bytes / x_tiles);
 }
 
 template <typename Math, typename Epi, int XR, int COLS>
@@ -899,7 +938,7 @@ void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, 
   static std::atomic<uint64_t> lds_set{0};
   if (!ensure_dynamic_lds(ctx, (const void*)kern, G::LDS_BYTES, lds_set)) return;
   const int64_t kts = K / G::K_STAGE;
-  const int splits = kn16_kwaves_splits(ctx, N, kts, COLS);
+  const int splits = kn16_kwaves_splits(ctx, N, kts, COLS, G::MT);
   hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN * splits)), dim3(256), G::LDS_BYTES,
                      ctx->stream, (int)M, (int)N, (int)kts, splits,
                      static_cast<const char*>(X), ldx_bytes, static_cast<const char*>(W),
@@ -907,7 +946,8 @@ void launch_kn16_kwaves_xr(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, 
                      reinterpret_cast<uint32_t*>(static_cast<char*>(ctx->workspace) +
                                                  ctx->ws_partial_bytes),
                      // one exchange word per pair of columns and row of x: 128 bytes per column
-                     (size_t)N * 128 <= ctx->ws_swap_bytes
+                     // and 32-row tile
+                     (size_t)N * 128 * G::MT <= ctx->ws_swap_bytes
                          ? reinterpret_cast<uint64_t*>(static_cast<char*>(ctx->workspace) +
                                                        ctx->ws_partial_bytes +
                                                        ctx->ws_counter_bytes)
@@ -926,15 +966,18 @@ void launch_kn16_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, con
     launch_kn16_kwaves_xr<Math, Epi, 8, COLS>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
   else if (M <= 16)
     launch_kn16_kwaves_xr<Math, Epi, 16, COLS>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
-  else
+  else if (M <= 32)
     launch_kn16_kwaves_xr<Math, Epi, 32, COLS>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+  else if constexpr (COLS == 128)  // two tiles of x: the rings only fit beside 4 KiB W pieces
+    launch_kn16_kwaves_xr<Math, Epi, 64, COLS>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
 }
 
 template <typename Geo>
 bool skinny_shape_ok(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K, int elem,
-                     const void* X, int64_t ldx, const void* W, int64_t ldw) {
+                     const void* X, int64_t ldx, const void* W, int64_t ldw,
+                     int64_t max_m = XROWS) {
   if (!ctx->workspace) return false;
-  if (M < 1 || M > XROWS || N <= 0 || K <= 0) return false;
+  if (M < 1 || M > max_m || N <= 0 || K <= 0) return false;
   if (N % Geo::BN || K % Geo::K_ELEMS) return false;
   if ((ldx * elem) % 16 || (ldw * elem) % 16) return false;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return false;
@@ -946,6 +989,21 @@ bool skinny_shape_ok(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K, 
 struct Slab32 {
   static constexpr int BN = 32, K_ELEMS = 128;
 };
+
+// 33 to 64 rows of x (two 32-row tiles per wave, x pieces half the size of the W pieces): the
+// K-over-the-waves kernel beats the tile kernel's 64-row tiles with split-K and a reduction launch
+// when its slabs x ranges put exactly one workgroup on every compute unit (M = 33 / 64, weights
+// rotated: N = K = 4096 14.5 / 16.1 against 17.5 / 19.3 us, N = K = 8192 30.0 / 33.4 against 35.0 /
+// 36.9, 32768 x 2048 26.3 / 28.0 against 30.0 / 31.5, 4096 x 11008 24.3 / 27.1 against 26.6 /
+// 29.5; int8 K x N 16384 x 4096 19.7 / 22.6 against 22.2 / 24.4), and loses where it does not
+// (11008 x 4096, 430 workgroups: 25.9 / 32.4 against 22.4 / 24.0; 28672 x 8192, 224: 85.3 /
+// 105.4 against 81.5 / 85.3; 13824 x 5120, 216: 32.4 / 40.2 against 29.8 / 32.5): the tile
+// kernel's smaller workgroups spread more evenly.  Forcing the family takes every shape.
+inline bool two_tiles_pay(const cigemmContext* ctx, int64_t slabs, int64_t kts, int cols) {
+  if (ctx->algo == CIGEMM_ALGO_SKINNY) return true;
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  return slabs * kn16_kwaves_splits(ctx, slabs * cols, kts, cols, 2) == cus;
+}
 
 // Which 16-bit decode kernel.  The K-over-the-waves kernel takes every shape it can (N and K
 // multiples of 64); the 256-column kernel with a barrier per stage is left with K a multiple of
@@ -961,9 +1019,14 @@ struct Slab32 {
 // 2048 k (2048 x 8192: 11.1 / 12.4 against 13.0 / 15.8 us, 8192 x 1024: 7.1 / 7.3 against 7.4 /
 // 8.8).
 // 0: neither, 1: 64-column slabs, 2: 256-column slabs with a barrier per stage, 3: 128-column slabs.
-inline int kn16_choice(const cigemmContext* ctx, int64_t N, int64_t K) {
+inline int kn16_choice(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K) {
   const bool kw_ok = N % 64 == 0 && K % 64 == 0 && (size_t)(N / 64) * 4 <= ctx->ws_counter_bytes;
   const bool sk_ok = N % GeoKN16<tile::MathBF16>::BN == 0 && K % GeoKN16<tile::MathBF16>::K_ELEMS == 0;
+  if (M > XROWS)  // 33 to 64 rows of x: two tiles, 128-column slabs only
+    return kw_ok && N % 128 == 0 && N / 128 >= 32 && K >= 2048 &&
+                   two_tiles_pay(ctx, N / 128, K / 64, 128)
+               ? 3
+               : 0;
   if (kw_ok && N % 128 == 0 && N / 128 >= 32 && K >= 2048 && N * K > (int64_t)4096 * 4096)
     return 3;
   if (kw_ok) return 1;
@@ -978,9 +1041,10 @@ template <typename Math, typename E16>
 const char* launch_skinny_16_on(cigemmContext* ctx, int64_t M, int64_t N, int64_t K,
                                 const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                                 uint16_t* C, int64_t ldc, bool bf16) {
-  const int which = kn16_choice(ctx, N, K);
+  const int which = kn16_choice(ctx, M, N, K);
   if (which == 3) {
     launch_kn16_kwaves<Math, 128>(ctx, M, N, K, A, lda * 2, B, ldb * 2, EpiStore16x4<E16>{C, ldc});
+    if (M > XROWS) return bf16 ? "bf16_skinny_64x128_kwaves" : "f16_skinny_64x128_kwaves";
     return bf16 ? "bf16_skinny_32x128_kwaves" : "f16_skinny_32x128_kwaves";
   }
   if (which == 1) {
@@ -1002,7 +1066,7 @@ struct Slab16Any {
 bool launch_skinny_16(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_t K,
                       const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, uint16_t* C,
                       int64_t ldc) {
-  if (!skinny_shape_ok<Slab16Any>(ctx, M, N, K, 2, A, lda, B, ldb)) return false;
+  if (!skinny_shape_ok<Slab16Any>(ctx, M, N, K, 2, A, lda, B, ldb, 2 * XROWS)) return false;
   if (ldc % 4 || ((uintptr_t)C & 7)) return false;
   const char* name =
       bf16 ? launch_skinny_16_on<tile::MathBF16, BF16>(ctx, M, N, K, A, lda, B, ldb, C, ldc, true)
@@ -1021,12 +1085,14 @@ struct SlabKN8 {
 static bool launch_skinny_i8_kn(cigemmContext* ctx, int64_t M, int64_t N, int64_t K,
                                 const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb,
                                 int32_t* C, int64_t ldc, const DequantArgs* dq) {
-  if (!skinny_shape_ok<SlabKN8>(ctx, M, N, K, 1, A, lda, B, ldb)) return false;
+  if (!skinny_shape_ok<SlabKN8>(ctx, M, N, K, 1, A, lda, B, ldb, 2 * XROWS)) return false;
+  if (M > XROWS && !two_tiles_pay(ctx, N / SlabKN8::BN, K / SlabKN8::K_ELEMS, SlabKN8::BN))
+    return false;
   if ((size_t)(N / SlabKN8::BN) * 4 > ctx->ws_counter_bytes) return false;
   if (!dq) {
     if (ldc % 4 || ((uintptr_t)C & 15)) return false;
     launch_kn16_kwaves<tile::MathI8, 128>(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32x4{C, ldc});
-    ctx->last_kernel = "i8_skinny_32x128_kwaves_kn";
+    ctx->last_kernel = M > XROWS ? "i8_skinny_64x128_kwaves_kn" : "i8_skinny_32x128_kwaves_kn";
     return true;
   }
   if (dq->out_bf16 ? (dq->ldo % 4 || ((uintptr_t)dq->out & 7))
@@ -1046,7 +1112,8 @@ static bool launch_skinny_i8_kn(cigemmContext* ctx, int64_t M, int64_t N, int64_
     if (dump) CIG_DQ(false, true); else CIG_DQ(false, false);
   }
 #undef CIG_DQ
-  ctx->last_kernel = "i8_skinny_32x128_kwaves_kn_dequant";
+  ctx->last_kernel =
+      M > XROWS ? "i8_skinny_64x128_kwaves_kn_dequant" : "i8_skinny_32x128_kwaves_kn_dequant";
   return true;
 }
 

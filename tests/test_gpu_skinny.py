@@ -225,6 +225,78 @@ def test_skinny_16bit_both_kernels_exact_inputs(handle, torch_gpu, oracle, rng, 
         assert (got[M:] == narrow(np.float32(7.0))).all()
 
 
+@pytest.mark.parametrize("kind", ["bf16", "f16"])
+@pytest.mark.parametrize("M,N,K,forced,expect", [
+    # one workgroup on every compute unit: 32 slabs x 8 ranges, 64 x 4 (counter exchange), 128 x 2
+    # (exchange words), 256 x 1 -> the decode kernel with two tiles of x
+    (33, 4096, 4096, False, "64x128_kwaves"), (64, 8192, 4096, False, "64x128_kwaves"),
+    (47, 16384, 2048, False, "64x128_kwaves"), (64, 32768, 2048, False, "64x128_kwaves"),
+    # any other grid: the tile kernel, unless the family is forced
+    (40, 11008, 4096, False, None), (64, 5120, 5120, False, None),
+    (40, 11008, 4096, True, "64x128_kwaves"), (64, 5120, 5120, True, "64x128_kwaves"),
+    (33, 13824, 2048, True, "64x128_kwaves"),
+])
+def test_skinny_16bit_two_tiles_of_x(handle, torch_gpu, oracle, rng, kind, M, N, K, forced, expect):
+    """33 to 64 rows of x: the K-over-the-waves kernel with two 32-row tiles per wave where its
+    grid is exactly one workgroup per compute unit (or when forced), bit-equal to the CPU loop on
+    exact-arithmetic inputs, three calls in a row over guard rows."""
+    torch = torch_gpu
+    if torch.cuda.get_device_properties(0).multi_processor_count != 256:
+        pytest.skip("the shapes assume 256 compute units")
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    narrow = oracle.f32_to_bf16 if kind == "bf16" else oracle.f32_to_f16
+    X, W = rng.choice(vals, size=(M, K)), rng.choice(vals, size=(K, N))
+    W[rng.random(size=W.shape) < 0.5] = 0
+    W[:, 128:256] = 0                      # a slab of zero sums (the exchange words' empty state)
+    want = narrow(oracle.gemm_f32(X, W))
+    fn = handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16
+    out = torch.full((M + 2, N), 7.0, dtype=torch.bfloat16 if kind == "bf16" else torch.float16, device="cuda")
+    x, w = to_dev(torch, narrow(X), kind), to_dev(torch, narrow(W), kind)
+    with handle.algo(ci.ALGO_SKINNY if forced else ci.ALGO_DEFAULT):
+        for _ in range(3):
+            fn(x, w, out=out[:M])
+            if expect:
+                assert handle.last_kernel == f"{kind}_skinny_{expect}", handle.last_kernel
+            else:
+                assert "skinny" not in handle.last_kernel, handle.last_kernel
+            got = bits(torch, out)
+            np.testing.assert_array_equal(got[:M], want)
+            assert (got[M:] == narrow(np.float32(7.0))).all()
+
+
+@pytest.mark.parametrize("M,N,K,forced", [(33, 8192, 8192, False), (64, 16384, 4096, False),
+                                          (50, 4096, 11008, False), (64, 11008, 4096, True),
+                                          (48, 4096, 2048, True)])
+def test_skinny_int8_kn_two_tiles_of_x(handle, torch_gpu, oracle, rng, M, N, K, forced):
+    """int8 K x N weights with 33 to 64 rows of x: raw accumulators and both dequantized output
+    types, bit for bit."""
+    torch = torch_gpu
+    if torch.cuda.get_device_properties(0).multi_processor_count != 256:
+        pytest.skip("the shapes assume 256 compute units")
+    X = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    W = rng.integers(-127, 128, size=(K, N), dtype=np.int8)
+    acc_ref = oracle.gemm_i8_i32(X, W, b_is_nk=False)
+    xd, wd = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda()
+    out = torch.full((M + 2, N + 4), -9, dtype=torch.int32, device="cuda")
+    sa = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
+    sb = rng.uniform(1e-3, 5e-2, N).astype(np.float32)
+    with handle.algo(ci.ALGO_SKINNY if forced else ci.ALGO_DEFAULT):
+        for _ in range(2):
+            handle.gemm_i8_i32(xd, wd, ci.B_KN, out=out[:M, :N])
+            assert handle.last_kernel == "i8_skinny_64x128_kwaves_kn", handle.last_kernel
+            o = out.cpu().numpy()
+            np.testing.assert_array_equal(o[:M, :N], acc_ref)
+            assert (o[M:] == -9).all() and (o[:, N:] == -9).all()
+        for out_type, ot in (("f32", ci.OUT_F32), ("bf16", ci.OUT_BF16)):
+            y, acc = handle.gemm_i8_dequant(xd, wd, torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda(),
+                                            ci.B_KN, ot, dump_acc=True)
+            assert handle.last_kernel == "i8_skinny_64x128_kwaves_kn_dequant", handle.last_kernel
+            np.testing.assert_array_equal(acc.cpu().numpy(), acc_ref)
+            expect = oracle.dequant(acc_ref, sa, sb, out_dtype=out_type, sa_per_row=True, sb_per_col=True)
+            got = bits(torch, y) if out_type == "bf16" else y.cpu().numpy()
+            np.testing.assert_array_equal(got, expect)
+
+
 @pytest.mark.parametrize("N,K,kernel", [(16384, 4096, "32x128"), (8192 - 64, 1024, "32x64")])
 @pytest.mark.parametrize("zero_part", ["all", "first_range", "second_range", "columns"])
 def test_two_range_exchange_with_zero_partial_sums(handle, torch_gpu, oracle, rng, zero_part, N, K, kernel):
