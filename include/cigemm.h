@@ -123,7 +123,9 @@ typedef enum cigemmAlgo {
   CIGEMM_ALGO_DEFAULT = -1,
   CIGEMM_ALGO_GENERIC = 0, /* any-shape scalar kernel (fp32: bit-exact with the CPU loop) */
   CIGEMM_ALGO_TILE = 1,    /* LDS-tiled MFMA kernel, 256-column tiles */
-  CIGEMM_ALGO_SKINNY = 2,  /* M <= 32 weight-streaming kernels (16-bit K x N, int8 N x K) */
+  CIGEMM_ALGO_SKINNY = 2,  /* weight-streaming decode kernels: M <= 32 (16-bit K x N, int8 N x K and
+                              K x N); M <= 64 for K x N weights of at least 4096 x 2048 in
+                              whole 128-column slabs */
   CIGEMM_ALGO_SMALL = 3,   /* fp32 32x32 tile per workgroup, k split over the waves */
   CIGEMM_ALGO_TILE_PAIRED = 4, /* LDS-tiled MFMA kernel with 128-row tiles, two workgroups resident
                               per compute unit and out of phase (16-bit, int8 K x N).  Never
