@@ -260,14 +260,14 @@ def k_sweep(torch, ci, wl, handle, steps, warmup):
 
 
 def decode_sweep(torch, ci, handle, steps, warmup):
-    """Decode GEMMs (M = 1 and 16) at layer shapes of common decoder models, bf16 K x N and int8
+    """Decode GEMMs (M = 1, 16 and 32) at layer shapes of common decoder models, bf16 K x N and int8
     N x K weights: microseconds per call and weight bytes per second.  Several weight buffers
     are rotated so that the Infinity Cache cannot serve them."""
     shapes = [(4096, 4096), (11008, 4096), (4096, 11008), (12288, 4096), (5120, 5120), (13824, 5120),
               (5120, 13824), (8192, 8192), (28672, 8192), (8192, 28672), (32000, 4096)]
     res = {}
     for (N, K) in shapes:
-        for M in (1, 16):
+        for M in (1, 16, 32):
             for kind in ("bf16", "int8"):
                 eb = 2 if kind == "bf16" else 1
                 nb = max(2, int(700e6 // (N * K * eb)) + 1)
@@ -317,7 +317,7 @@ def main():
                     help="instead of the benchmark: time the tile kernel at several K per M x N and "
                          "fit its fixed cost per tile and its cost per stage")
     ap.add_argument("--decode-sweep", action="store_true",
-                    help="instead of the benchmark: decode GEMMs (M = 1, 16) at layer shapes of common "
+                    help="instead of the benchmark: decode GEMMs (M = 1, 16, 32) at layer shapes of common "
                          "decoder models, bf16 and int8")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
