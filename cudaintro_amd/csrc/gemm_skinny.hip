@@ -473,19 +473,37 @@ struct NK8KW {
   static constexpr int DPS = 4 + XR / 8;             // per wave and stage, 1 KiB each
 };
 
-template <typename Epi, int XR, bool DEEP>
+template <typename Epi, int XR, bool DEEP, bool ROW_TILES>
 __global__ __launch_bounds__(256, 2) void skinny_nk8_kwaves_kernel(int M, int N, int K,
                                                                    const char* __restrict__ X,
                                                                    int64_t ldx,
                                                                    const char* __restrict__ W,
-                                                                   int64_t ldw, Epi epi) {
+                                                                   int64_t ldw, Epi epi,
+                                                                   int row_tiles) {
   typedef tile::MathI8 Math;
   typedef NK8KW<XR, DEEP> G;
   constexpr int NS = G::NSTAGES, DIST = NS - 1;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int t = threadIdx.x, l = t & 63;
   const int w = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int64_t n0 = (int64_t)blockIdx.x * G::BN;
+  // With several row tiles the grid is that many times the slabs: rows 0 .. XR - 1, XR .. 2 XR - 1,
+  // ... of x go to different workgroups, which the block order puts on the same XCD (blocks b,
+  // b + 8, ...) and close in time, so that the later ones find the slab's weight rows in that
+  // XCD's L2.
+  int slab = blockIdx.x, m_base = 0;
+  if constexpr (ROW_TILES) {
+    if (gridDim.x % (8 * row_tiles) == 0) {
+      m_base = ((blockIdx.x >> 3) % row_tiles) * XR;
+      slab = blockIdx.x / (8 * row_tiles) * 8 + (blockIdx.x & 7);
+    } else {
+      m_base = (blockIdx.x % row_tiles) * XR;
+      slab = blockIdx.x / row_tiles;
+    }
+    if (m_base >= M) return;  // (a tile past the last row: nothing to do)
+    X += (int64_t)m_base * ldx;
+    M = M - m_base < XR ? M - m_base : XR;
+  }
+  const int64_t n0 = (int64_t)slab * G::BN;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
   // K is a multiple of 128: the last stage may hold fewer than four k-chunks
   const int KTS = (K + G::K_ELEMS - 1) / G::K_ELEMS;
@@ -504,7 +522,7 @@ __global__ __launch_bounds__(256, 2) void skinny_nk8_kwaves_kernel(int M, int N,
   // Workgroups start at different stages of K and wrap around (integer sums do not depend on
   // the order): at any moment they read different 512-byte columns of their rows, which spreads
   // the requests over the memory channels (19.4 -> 14.1 us per call at N = K = 8192).
-  const int rot = (int)((blockIdx.x * 7u) % (unsigned)KTS);
+  const int rot = (int)(((unsigned)slab * 7u) % (unsigned)KTS);
   // first k of wave w's chunk of the s-th stage this workgroup visits, or -1 when that chunk
   // lies past K (last stage of a K that is not a multiple of 512)
   auto chunk_k = [&](int s) {
@@ -579,7 +597,7 @@ __global__ __launch_bounds__(256, 2) void skinny_nk8_kwaves_kernel(int M, int N,
     const i32x4 p = *reinterpret_cast<const i32x4*>(red + (ww * 32 + m) * RLD + c);
     sum += p;
   }
-  epi(m, n0 + c, sum[0], sum[1], sum[2], sum[3]);
+  epi(m + m_base, n0 + c, sum[0], sum[1], sum[2], sum[3]);
 }
 
 template <typename Epi, int XR, bool DEEP>
@@ -589,12 +607,27 @@ void launch_skinny_kwaves_ring(cigemmContext* ctx, int64_t M, int64_t N, int64_t
   typedef NK8KW<XR, DEEP> G;
   constexpr int LDS_BYTES = G::NSTAGES * G::STAGE_BYTES;
   static_assert(LDS_BYTES * (DEEP ? 1 : 2) <= 160 * 1024, "rings must fit the LDS");
-  auto kern = skinny_nk8_kwaves_kernel<Epi, XR, DEEP>;
+  auto kern = skinny_nk8_kwaves_kernel<Epi, XR, DEEP, false>;
   static std::atomic<uint64_t> lds_set{0};
   if (!ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set)) return;
   hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN)), dim3(256), LDS_BYTES, ctx->stream, (int)M,
                      (int)N, (int)K, static_cast<const char*>(X), ldx_bytes,
-                     static_cast<const char*>(W), ldw_bytes, epi);
+                     static_cast<const char*>(W), ldw_bytes, epi, 1);
+}
+
+// the same with the rows of x cut into `row_tiles` tiles of XR rows (nk8_row_tiles)
+template <typename Epi, int XR>
+void launch_skinny_kwaves_row_tiles(cigemmContext* ctx, int64_t M, int64_t N, int64_t K,
+                                    const void* X, int64_t ldx_bytes, const void* W,
+                                    int64_t ldw_bytes, const Epi& epi, int row_tiles) {
+  typedef NK8KW<XR, false> G;
+  constexpr int LDS_BYTES = G::NSTAGES * G::STAGE_BYTES;
+  auto kern = skinny_nk8_kwaves_kernel<Epi, XR, false, true>;
+  static std::atomic<uint64_t> lds_set{0};
+  if (!ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set)) return;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(N / G::BN * row_tiles)), dim3(256), LDS_BYTES,
+                     ctx->stream, (int)M, (int)N, (int)K, static_cast<const char*>(X), ldx_bytes,
+                     static_cast<const char*>(W), ldw_bytes, epi, row_tiles);
 }
 
 template <typename Epi, int XR>
@@ -608,6 +641,20 @@ void launch_skinny_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, c
     }
   }
   launch_skinny_kwaves_ring<Epi, XR, false>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+}
+
+// Few slabs and more than 8 rows of x: the rows are cut into tiles of 8 (or 16) and every tile
+// gets workgroups of its own, as long as all of them find a compute unit -- a slab's weights
+// then cross the fabric once and are read from the XCD's L2 by the other tiles.  One workgroup
+// per slab leaves most of the chip idle here and moves as many bytes of x as of W at 32 rows
+// (weights rotated, us per call: 4096 x 11008 M = 16 13.9 -> 12.5, M = 32 17.1 -> 13.5;
+// 2048 x 8192 M = 32 12.3 -> 8.9 with four tiles of 8, 9.8 with two of 16; with more workgroups
+// than units it loses: 5120 x 5120 M = 32 10.3 -> 12.8, 3072 x 8192 in four tiles 12.8 -> 14.4).
+// Returns the number of row tiles for tiles of `xr` rows, 0 when that does not apply.
+inline int nk8_row_tiles(const cigemmContext* ctx, int64_t M, int64_t N, int xr) {
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  const int64_t slabs = N / 32, tiles = (M + xr - 1) / xr;
+  return tiles > 1 && slabs % 8 == 0 && slabs * tiles <= cus ? (int)tiles : 0;
 }
 
 // (A variant with 1024-byte stages, each wave moving 256 contiguous bytes of every weight row --
@@ -628,6 +675,10 @@ bool launch_skinny_nk8(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, cons
   if (N / 32 >= cus / 4 || K <= 16384 || N % GeoNK8::BN) {
     if (M <= 8)
       launch_skinny_kwaves<Epi, 8>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
+    else if (const int t8 = nk8_row_tiles(ctx, M, N, 8))
+      launch_skinny_kwaves_row_tiles<Epi, 8>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi, t8);
+    else if (const int t16 = nk8_row_tiles(ctx, M, N, 16))
+      launch_skinny_kwaves_row_tiles<Epi, 16>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi, t16);
     else if (M <= 16)
       launch_skinny_kwaves<Epi, 16>(ctx, M, N, K, X, ldx_bytes, W, ldw_bytes, epi);
     else

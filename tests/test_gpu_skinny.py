@@ -99,7 +99,9 @@ def test_skinny_int8_nk(handle, torch_gpu, oracle, rng, M, N, K, out_type):
 @pytest.mark.parametrize("N,K", [(8192, 512), (8192 + 128, 1536), (8192, 4096 + 128), (128, 128), (256, 640),
                                  (32, 256), (8192 + 96, 1024), (160, 16384 + 640),
                                  (2048, 16384 + 384), (256, 16384 + 512), (1024, 32768 + 128),
-                                 (11008, 1024)])
+                                 (11008, 1024),
+                                 # few slabs: rows of x in tiles of 8 or 16 with workgroups of their own
+                                 (2048, 1536), (4096, 1152), (1024, 2048 + 128)])
 def test_skinny_int8_without_split_k(handle, torch_gpu, oracle, rng, M, N, K):
     """The kernel that splits K over the waves of a workgroup instead of over workgroups, with
     8, 16 or 32 rows of x per stage and a last stage of one to four k-chunks.  A few slabs of
