@@ -757,8 +757,9 @@ __global__ __launch_bounds__(256, 2) void skinny_kn16_kwaves_kernel(
   const int64_t n0 = (int64_t)slab * G::BN;
   // K range `split` of `splits`: stages [split * stages / splits, (split + 1) * stages / splits),
   // as even as the stage count allows; this wave's k rows of its first stage
-  const int s_begin = (int)((int64_t)split * stages / splits);
-  const int KTS = (int)((int64_t)(split + 1) * stages / splits) - s_begin;
+  // (32-bit: split < 16 and stages < 2^25, and a 64-bit division costs a few hundred cycles)
+  const int s_begin = (int)((unsigned)(split * stages) / (unsigned)splits);
+  const int KTS = (int)((unsigned)((split + 1) * stages) / (unsigned)splits) - s_begin;
   const int64_t k0 = (int64_t)s_begin * G::K_STAGE + G::KW * w;
   char* const wave_lds = lds + w * G::WAVE_BYTES;
   const uint32_t wave_base =
