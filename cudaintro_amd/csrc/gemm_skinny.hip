@@ -652,9 +652,7 @@ void launch_skinny_kwaves(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, c
 // than units it loses: 5120 x 5120 M = 32 10.3 -> 12.8, 3072 x 8192 in four tiles 12.8 -> 14.4).
 // Returns the number of row tiles for tiles of `xr` rows, 0 when that does not apply.
 inline int nk8_row_tiles(const cigemmContext* ctx, int64_t M, int64_t N, int xr) {
-  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-  const int64_t slabs = N / 32, tiles = (M + xr - 1) / xr;
-  return tiles > 1 && slabs % 8 == 0 && slabs * tiles <= cus ? (int)tiles : 0;
+  return skinny_plan::nk8_row_tiles(M, N, xr, ctx->num_cus);
 }
 
 // (A variant with 1024-byte stages, each wave moving 256 contiguous bytes of every weight row --
@@ -1053,8 +1051,8 @@ struct Slab32 {
 // kernel's smaller workgroups spread more evenly.  Forcing the family takes every shape.
 inline bool two_tiles_pay(const cigemmContext* ctx, int64_t slabs, int64_t kts, int cols) {
   if (ctx->algo == CIGEMM_ALGO_SKINNY) return true;
-  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-  return slabs * kn16_kwaves_splits(ctx, slabs * cols, kts, cols, 2) == cus;
+  return skinny_plan::two_tiles_fit(slabs, kts, cols, ctx->num_cus, ctx->ws_counter_bytes,
+                                    ctx->ws_partial_bytes);
 }
 
 // Which 16-bit decode kernel.  The K-over-the-waves kernel takes every shape it can (N and K

@@ -34,5 +34,24 @@ inline int kwaves_splits(int64_t slabs, int64_t stages, int cols, int cus, size_
   return best;
 }
 
+// int8 N x K weights in 32-row slabs, few slabs and more than `xr` rows of x: the rows are cut into
+// tiles of `xr` rows (8 or 16) that get workgroups of their own, as long as every workgroup
+// still finds a compute unit and the slabs come in whole groups of 8 (the block order then
+// puts the tiles of a slab on one XCD, whose L2 serves the slab's weights to all but the first).
+// Returns the number of tiles, 0 when that does not apply.
+inline int nk8_row_tiles(int64_t M, int64_t N, int xr, int cus) {
+  if (cus <= 0) cus = 256;
+  const int64_t slabs = N / 32, tiles = (M + xr - 1) / xr;
+  return tiles > 1 && slabs % 8 == 0 && slabs * tiles <= cus ? (int)tiles : 0;
+}
+
+// K x N weights with 33 to 64 rows of x (two 32-row tiles per wave): taken when slabs x K ranges
+// put exactly one workgroup on every compute unit.
+inline bool two_tiles_fit(int64_t slabs, int64_t stages, int cols, int cus, size_t counter_bytes,
+                          size_t partial_bytes) {
+  if (cus <= 0) cus = 256;
+  return slabs * kwaves_splits(slabs, stages, cols, cus, counter_bytes, partial_bytes / 2) == cus;
+}
+
 }  // namespace skinny_plan
 }  // namespace cig

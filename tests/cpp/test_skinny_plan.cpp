@@ -7,6 +7,8 @@
 #include "skinny_plan.h"
 
 using cig::skinny_plan::kwaves_splits;
+using cig::skinny_plan::nk8_row_tiles;
+using cig::skinny_plan::two_tiles_fit;
 
 static int failures = 0;
 #define EXPECT(cond)                                                     \
@@ -42,6 +44,26 @@ int main() {
   EXPECT(kwaves_splits(64, 128, 128, 256, counters, (size_t)3 * 64 * 128 * 128) == 3);
   // a device that does not report its units counts as 256
   EXPECT(kwaves_splits(64, 128, 128, 0, counters, partials) == 4);
+
+  // rows of x in tiles for int8 N x K weights with few slabs
+  EXPECT(nk8_row_tiles(32, 4096, 8, 256) == 0);    // 128 slabs x 4 tiles > 256 units
+  EXPECT(nk8_row_tiles(32, 4096, 16, 256) == 2);
+  EXPECT(nk8_row_tiles(16, 4096, 8, 256) == 2);
+  EXPECT(nk8_row_tiles(8, 4096, 8, 256) == 0);     // one tile: nothing to cut
+  EXPECT(nk8_row_tiles(32, 2048, 8, 256) == 4);
+  EXPECT(nk8_row_tiles(20, 2048, 8, 256) == 3);
+  EXPECT(nk8_row_tiles(32, 5120, 16, 256) == 0);   // 160 slabs x 2 > 256
+  EXPECT(nk8_row_tiles(32, 2048 + 32, 8, 256) == 0);  // 65 slabs: not in groups of 8
+  EXPECT(nk8_row_tiles(32, 2048, 8, 0) == 4);
+  // 33 to 64 rows of x: exactly one workgroup per unit
+  EXPECT(two_tiles_fit(4096 / 128, 4096 / 64, 128, 256, counters, partials));
+  EXPECT(two_tiles_fit(8192 / 128, 8192 / 64, 128, 256, counters, partials));
+  EXPECT(two_tiles_fit(16384 / 128, 4096 / 64, 128, 256, counters, partials));
+  EXPECT(two_tiles_fit(32768 / 128, 2048 / 64, 128, 256, counters, partials));
+  EXPECT(!two_tiles_fit(11008 / 128, 4096 / 64, 128, 256, counters, partials));
+  EXPECT(!two_tiles_fit(28672 / 128, 8192 / 64, 128, 256, counters, partials));
+  EXPECT(!two_tiles_fit(13824 / 128, 5120 / 64, 128, 256, counters, partials));
+  EXPECT(!two_tiles_fit(5120 / 128, 5120 / 64, 128, 256, counters, partials));
 
   // invariants over a sweep
   long checked = 0;
