@@ -188,7 +188,7 @@ def cpu_rows_baseline(run_rows, M, ops_per_row, unit, what, target_seconds=3.0):
             "kind": "port", "sample": f"first {rows2} of {M} rows of the same problem, {what}, {dt:.2f} s"}, res
 
 
-def k_sweep(torch, ci, wl, handle, steps, warmup):
+def k_sweep(torch, ci, wl, probe, handle, steps, warmup):
     """Per-launch time of the tile kernel at several K for a fixed M x N, and the least-squares
     fit t = rounds * (a + b * stages): `a` is what one output tile costs whatever its K
     (pipeline fill, epilogue, the burst of output stores), `b` the cost of one 64-byte stage
@@ -252,7 +252,7 @@ def k_sweep(torch, ci, wl, handle, steps, warmup):
                 b = torch.randn((4096, No), device="cuda").to(torch.bfloat16)
                 o = torch.empty((Mo, No), dtype=torch.bfloat16, device="cuda")
             for _ in range(20):
-                ph = handle.probe_tile_phases(a, b, o)
+                ph = probe.tile_phases(handle, a, b, o)
             occ[f"{kind}_{Mo}x{No}x4096"] = ph
             log(f"[occupancy] {kind} {Mo}x{No}x4096: {json.dumps(ph)}")
             del a, b, o
@@ -327,6 +327,7 @@ def main():
 
     import torch
     import cudaintro_amd as ci
+    from cudaintro_amd import probe
     from cudaintro_amd import workloads as wl
 
     if not torch.cuda.is_available():
@@ -334,7 +335,7 @@ def main():
         sys.exit(1)
     handle = ci.Handle()
     if args.k_sweep:
-        k_sweep(torch, ci, wl, handle, args.steps, args.warmup)
+        k_sweep(torch, ci, wl, probe, handle, args.steps, args.warmup)
         return
     if args.decode_sweep:
         decode_sweep(torch, ci, handle, args.steps, args.warmup)
@@ -369,7 +370,7 @@ def main():
     # where the time of one launch goes, from timestamps inside the kernel (one instrumented
     # launch of the same kernel, taken while the chip is in the state the timed loop left)
     for _ in range(3):
-        phases = handle.probe_tile_phases(A, B, C)
+        phases = probe.tile_phases(handle, A, B, C)
     roofline["phases"] = phases
     roofline["clock_ghz_main_loop_this_run"] = phases["main_loop_clock_ghz"]
     # matrix-core issue cycles of one 64-byte stage of the 256 x 256 tile: 32 instructions of 8
@@ -379,28 +380,40 @@ def main():
                                                   max(50, args.steps))
     # HBM-side bytes per launch and the counter decomposition of the same kernel are not
     # measurable from inside this process: they come from the rocprofv3 --pmc runs of this
-    # same command summarised in profiles/ (the file says which runs).
+    # same command summarised in profiles/ (the file says which runs).  Everything copied from
+    # there sits under `from_profiles`, apart from `traffic`, whose source is named beside it.
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(traffic_file):
-        prof = json.load(open(traffic_file))
+    prof = json.load(open(traffic_file)) if os.path.exists(traffic_file) else {}
+    if prof:
         roofline["traffic"] = prof.get(f"bf16_{n}")
         roofline["traffic_source"] = "profiles/hbm_traffic.json"
-        for key in ("mfma_busy", "clock_ghz"):
-            if f"bf16_{n}_{key}" in prof:
-                roofline[key] = prof[f"bf16_{n}_{key}"]
-                roofline[key + "_source"] = "profiles/hbm_traffic.json"
+        roofline["from_profiles"] = {key: prof[f"bf16_{n}_{key}"] for key in ("mfma_busy", "clock_ghz")
+                                     if f"bf16_{n}_{key}" in prof}
+        roofline["from_profiles"]["source"] = "profiles/hbm_traffic.json (rocprofv3 --pmc runs, not this run)"
+
     # What a register-resident loop of the same matrix instruction sustains in this run on
     # random operand bits, with no memory traffic at all: the chip is power limited on such
     # data, so this, not the datasheet peak, is the ceiling a kernel can approach.
-    ops_box = [0]
+    def sustained(kind):
+        ops_box = [0]
 
-    def fn_probe():
-        ops_box[0] = handle.probe_mfma("bf16", True, 20000)
-    _, e_probe = time_calls(torch, fn_probe, 20, 10)
-    roofline["sustained_peak"] = ops_box[0] * 20 / e_probe / 1e12
+        def fn_probe():
+            ops_box[0] = probe.mfma(handle, kind, True, 20000)
+        _, e_probe = time_calls(torch, fn_probe, 20, 10)
+        return ops_box[0] * 20 / e_probe / 1e12
+
+    roofline["sustained_peak"] = sustained("bf16")
     roofline["sustained_peak_what"] = ("register-resident v_mfma_f32_32x32x16_bf16 loop, random "
                                        "operand bits, one wave per SIMD, same run")
     roofline["frac_of_sustained"] = achieved / roofline["sustained_peak"]
+    # The metric is quoted per dtype: bf16, fp16 and int8 at n^3, each against its datasheet peak
+    # and against what the register-resident loop of its matrix instruction sustained in this run.
+    per_dtype = {"bf16": {"achieved": achieved, "unit": "TFLOP/s", "peak": PEAK_16BIT_TFLOPS,
+                          "frac": achieved / PEAK_16BIT_TFLOPS, "sustained_peak": roofline["sustained_peak"],
+                          "frac_of_sustained": roofline["frac_of_sustained"], "kernel": kernel,
+                          "ms": ev / args.steps * 1e3, "cycles_per_stage": phases["cycles_per_stage"],
+                          "clock_ghz_main_loop": phases["main_loop_clock_ghz"]}}
+    roofline["per_dtype"] = per_dtype
 
     cpu = None
     if not args.no_cpu:
@@ -417,25 +430,35 @@ def main():
             fn = handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16
             w, e = time_calls(torch, lambda: fn(a, b, out=c), args.steps, args.warmup)
             t = ops * args.steps / e / 1e12
-            return {"tflops": t, "frac_of_peak": t / PEAK_16BIT_TFLOPS, "peak": PEAK_16BIT_TFLOPS,
-                    "ms": e / args.steps * 1e3, "kernel": handle.last_kernel}
+            res = {"tflops": t, "frac_of_peak": t / PEAK_16BIT_TFLOPS, "peak": PEAK_16BIT_TFLOPS,
+                   "ms": e / args.steps * 1e3, "kernel": handle.last_kernel}
+            for _ in range(3):
+                res["phases"] = probe.tile_phases(handle, a, b, c)
+            return res
 
         log(f"[bench] fp16 {n}^3")
-        per_config[f"fp16_{n}"] = run16("f16")
+        r16 = run16("f16")
+        per_config[f"fp16_{n}"] = r16
+        sp = sustained("f16")
+        per_dtype["fp16"] = {"achieved": r16["tflops"], "unit": "TFLOP/s", "peak": PEAK_16BIT_TFLOPS,
+                             "frac": r16["frac_of_peak"], "sustained_peak": sp,
+                             "frac_of_sustained": r16["tflops"] / sp, "kernel": r16["kernel"], "ms": r16["ms"],
+                             "cycles_per_stage": r16["phases"]["cycles_per_stage"],
+                             "clock_ghz_main_loop": r16["phases"]["main_loop_clock_ghz"]}
+        log(f"[bench] fp16 {n}^3: {json.dumps(per_dtype['fp16'])}")
 
         # The same headline problem on the two-workgroups-per-unit form of the tile kernel
-        # (CIGEMM_ALGO_TILE_PAIRED, never chosen by default): more matrix instructions issued
+        # (libcigemm_probe.so; the library never chooses it): more matrix instructions issued
         # per cycle, a lower clock under the power limit.  Recorded as the measured reason for
         # the default's choice.
         a_b, b_b = wl.normal_16bit(n, n, n, seed=2, kind="bf16")
         a, b = dev16(torch, a_b, "bf16"), dev16(torch, b_b, "bf16")
         c = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
-        with handle.algo(ci.ALGO_TILE_PAIRED):
-            w, e = time_calls(torch, lambda: handle.gemm_bf16(a, b, out=c), args.steps, args.warmup)
-            name_p = handle.last_kernel
+        w, e = time_calls(torch, lambda: probe.gemm16_paired(handle, a, b, out=c), args.steps, args.warmup)
+        name_p = handle.last_kernel
         t = ops * args.steps / e / 1e12
         for _ in range(3):
-            ph = handle.probe_tile_phases(a, b, c, paired=True)
+            ph = probe.tile_phases(handle, a, b, c, paired=True)
         per_config[f"bf16_{n}_two_workgroups_per_unit"] = {
             "tflops": t, "frac_of_peak": t / PEAK_16BIT_TFLOPS, "peak": PEAK_16BIT_TFLOPS,
             "ms": e / args.steps * 1e3, "ms_over_default": e / args.steps / (ev / args.steps),
@@ -514,7 +537,7 @@ def main():
                 # output element as the fp32 dequantized one)
                 o32 = out if not dequant else torch.empty((M, N), dtype=torch.int32, device="cuda")
                 for _ in range(3):
-                    ph = handle.probe_tile_phases(a, b, o32)
+                    ph = probe.tile_phases(handle, a, b, o32)
                 per_config[name]["phases_raw_i32_out"] = ph
                 del o32
             if not args.no_cpu:
@@ -546,7 +569,24 @@ def main():
             Xq, sx, Wq, sw = wl.quantized_linear(2048, 4096, 11008, seed=3)
             return Xq, Wq, sx, sw, ci.B_NK, ci.OUT_BF16
 
+        def mk_square_nk(sz, seed):
+            def f():
+                Aq, Bq, sa, sb = wl.int8_uniform(sz, sz, sz, seed=seed)
+                return Aq, np.ascontiguousarray(Bq.T), sa, sb, ci.B_NK, ci.OUT_F32
+            return f
+
         run_i8(f"int8_{n}_raw_i32", n, n, n, mk_square(n, 1), False)
+        r8 = per_config[f"int8_{n}_raw_i32"]
+        sp = sustained("i8")
+        per_dtype["int8"] = {"achieved": r8["tops"], "unit": "TOP/s", "peak": PEAK_INT8_TOPS,
+                             "frac": r8["frac_of_peak"], "sustained_peak": sp,
+                             "frac_of_sustained": r8["tops"] / sp, "kernel": r8["kernel"], "ms": r8["ms"],
+                             "cycles_per_stage": r8["phases_raw_i32_out"]["cycles_per_stage"],
+                             "clock_ghz_main_loop": r8["phases_raw_i32_out"]["main_loop_clock_ghz"]}
+        log(f"[bench] int8 {n}^3: {json.dumps(per_dtype['int8'])}")
+        # the same problem with the weights stored N x K (each output channel contiguous: the
+        # layout of the quantized linear layer)
+        run_i8(f"int8_{n}_nk_raw_i32", n, n, n, mk_square_nk(n, 1), False)
         run_i8("int8_4096_dequant_f32", 4096, 4096, 4096, mk_square(4096, 1), True)
         run_i8("int8_linear_2048x11008x4096_dequant_bf16", 2048, 11008, 4096, mk_linear, True)
 
@@ -599,6 +639,17 @@ def main():
                                                     "peak": PEAK_HBM_GBS, "us": e / args.steps * 1e6,
                                                     "bytes": fb.numel() * 2}
         del fb
+        # C2 is one round of tiles whose 64 MiB of fp32 output all units store at the same time,
+        # with the matrix cores idle: its floor on this chip is the main loop plus the output's
+        # bytes at the rate the fill kernel (a pure store stream) reached in this run.
+        c2 = per_config["int8_4096_dequant_f32"]
+        out_bytes = 4096 * 4096 * 4
+        floor_us = c2["phases_raw_i32_out"]["main_loop_us"] + out_bytes / (gbs * 1e9) * 1e6
+        c2["floor_us"] = floor_us
+        c2["floor_what"] = ("main loop of the instrumented launch + 64 MiB of output at the fill kernel's "
+                            "write rate of this run")
+        c2["frac_of_floor"] = floor_us / (c2["ms"] * 1e3)
+        c2["floor_tops"] = wl.gemm_ops(4096, 4096, 4096) / floor_us / 1e6
         for rows_q, cols_q in ((2048, 4096), (8192, 8192)):
             xq_ = torch.from_numpy(r.standard_normal((rows_q, cols_q)).astype(np.float32)).cuda()
             outq = (torch.empty((rows_q, cols_q), dtype=torch.int8, device="cuda"),
@@ -731,19 +782,62 @@ def main():
 
         # What the matrix cores sustain with no memory traffic at all, at the clock the chip
         # holds under that load, on constant and on random operand bits.
-        probe = {}
+        probe_res = {}
         for kind in ("bf16", "f16", "i8", "f32"):
             for rnd in (False, True):
                 ops_box = [0]
 
                 def fnp():
-                    ops_box[0] = handle.probe_mfma(kind, rnd, 5000 if kind == "f32" else 20000)
+                    ops_box[0] = probe.mfma(handle, kind, rnd, 5000 if kind == "f32" else 20000)
                 w, e = time_calls(torch, fnp, 20, 10)
-                probe[f"{kind}_{'random' if rnd else 'constant'}_bits"] = ops_box[0] * 20 / e / 1e12
-        mfma_probe.update(probe)
+                probe_res[f"{kind}_{'random' if rnd else 'constant'}_bits"] = ops_box[0] * 20 / e / 1e12
+        mfma_probe.update(probe_res)
+        # What the other instructions of the tile kernel's stage cost in matrix-core issue time:
+        # cycles per 32 matrix instructions (1024 when nothing delays them) with n LDS-DMA
+        # instructions, the stage's 24 LDS fragment reads and its barrier added, all units busy.
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        issue = {}
+        for n_dma, n_lds, bar in ((0, 0, 0), (2, 0, 0), (4, 0, 0), (8, 0, 0), (0, 24, 0), (0, 0, 1),
+                                  (8, 24, 0), (8, 24, 1)):
+            for _ in range(2):
+                r_ic = probe.issue_cost(handle, n_dma, n_lds, bool(bar), cus, 4000)
+            issue[f"dma{n_dma}_lds{n_lds}_bar{bar}"] = round(r_ic["cycles_per_stage"], 1)
+        one = probe.issue_cost(handle, 8, 24, True, 1, 4000)
+        issue["dma8_lds24_bar1_one_workgroup"] = round(one["cycles_per_stage"], 1)
+        mfma_probe["issue_cost_cycles_per_stage"] = issue
+        roofline["issue_ceiling"] = 1024.0 / issue["dma8_lds24_bar1"]
+        roofline["issue_ceiling_what"] = ("1024 matrix-core issue cycles per stage / cycles per stage of a "
+                                          "register-resident loop with the stage's 8 LDS-DMA instructions, 24 "
+                                          "LDS fragment reads and barrier, same run")
         for k, v in per_config.items():
             log(f"[bench]   {k}: {json.dumps(v)}")
-        log(f"[bench]   register-resident MFMA loop, T(FL)OP/s: {json.dumps(probe)}")
+        log(f"[bench]   register-resident MFMA loop, T(FL)OP/s: {json.dumps(probe_res)}")
+        log(f"[bench]   issue cost, cycles per stage: {json.dumps(issue)}")
+
+    # The line printed last holds the figures; the full per-configuration records (phases, CPU
+    # baselines, samples) were logged above.  One entry per configuration: value, unit, fraction
+    # of its roofline, time per call, kernel.
+    def compact(v):
+        if not isinstance(v, dict) or not any(k in v for k in ("tflops", "tops", "gbs")):
+            return v
+        key = "tflops" if "tflops" in v else "tops" if "tops" in v else "gbs"
+        out = {"value": round(v[key], 2), "unit": {"tflops": "TFLOP/s", "tops": "TOP/s", "gbs": "GB/s"}[key],
+               "frac_of_peak": round(v["frac_of_peak"], 4)}
+        us = v["us"] if "us" in v else v["ms"] * 1e3
+        out["us"] = round(us, 2)
+        if "kernel" in v:
+            out["kernel"] = v["kernel"]
+        for extra in ("us_replayed_from_graph", "ms_over_default", "ms_over_aligned", "scalar_kernel_tflops",
+                      "floor_us", "frac_of_floor", "cpu_gflops"):
+            if extra in v:
+                out[extra] = round(v[extra], 4)
+        base = v.get("cpu_baseline")
+        if base:
+            out["cpu"] = {"value": float(f"{base['value']:.4g}"), "unit": base["unit"], "cores": base["cores"]}
+            for flag in ("gpu_rows_bit_exact",):
+                if flag in base:
+                    out["cpu"][flag] = base[flag]
+        return out
 
     line = {
         "metric": "GEMM TFLOPS/TOPS at 8192^3 per dtype (int8/bf16/fp16) + % of MFMA peak",
@@ -762,9 +856,28 @@ def main():
                                "bf16 out, row-major", "M": n, "N": n, "K": n},
         "roofline": roofline,
         "cpu_baseline": cpu,
-        "per_config": per_config,
-        "mfma_only_probe": mfma_probe,
     }
+    # the metric's three dtypes, flat (beside roofline.per_dtype)
+    for dt, rec in per_dtype.items():
+        unit = "tflops" if dt != "int8" else "tops"
+        line[f"{dt}_{n}_{unit}"] = rec["achieved"]
+        line[f"{dt}_{n}_frac_of_peak"] = rec["frac"]
+        line[f"{dt}_{n}_frac_of_sustained"] = rec["frac_of_sustained"]
+        roofline[f"{dt}_{n}_achieved"] = rec["achieved"]
+        roofline[f"{dt}_{n}_frac"] = rec["frac"]
+    line["per_config"] = {k: compact(v) for k, v in per_config.items()}
+    line["mfma_only_probe"] = mfma_probe
+    # the BASELINE configurations once more, last on stderr
+    for dt, rec in per_dtype.items():
+        log(f"[bench] C3/{dt} {n}^3: {rec['achieved']:.1f} {rec['unit']} = {rec['frac'] * 100:.1f} % of "
+            f"{rec['peak']:.1f}, {rec['frac_of_sustained'] * 100:.1f} % of the {rec['sustained_peak']:.0f} the chip "
+            f"sustains on random bits; {rec['ms']:.4f} ms, {rec['kernel']}")
+    for tag, key in (("C1", "fp32_512"), ("C2", "int8_4096_dequant_f32"),
+                     ("C4", "int8_linear_2048x11008x4096_dequant_bf16"),
+                     ("C5", "skinny_bf16_M1"), ("C5", "skinny_bf16_M8"), ("C5", "skinny_bf16_M32"),
+                     ("C5", "skinny_int8_M1"), ("C5", "skinny_int8_M8"), ("C5", "skinny_int8_M32")):
+        if key in per_config:
+            log(f"[bench] {tag} {key}: {json.dumps(compact(per_config[key]))}")
     print(json.dumps(line), flush=True)
 
 

@@ -14,7 +14,6 @@ from .cigemm import (  # noqa: F401
     ALGO_SKINNY,
     ALGO_SMALL,
     ALGO_TILE,
-    ALGO_TILE_PAIRED,
     ALGO_MFMA_ANY,
     B_KN,
     B_NK,

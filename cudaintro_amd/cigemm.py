@@ -17,7 +17,7 @@ _SUITE = os.path.join(_HERE, "gemm_suite")
 
 B_KN, B_NK = 0, 1
 ACT_NONE, ACT_RELU = 0, 1
-ALGO_DEFAULT, ALGO_GENERIC, ALGO_TILE, ALGO_SKINNY, ALGO_SMALL, ALGO_TILE_PAIRED, ALGO_MFMA_ANY = -1, 0, 1, 2, 3, 4, 5
+ALGO_DEFAULT, ALGO_GENERIC, ALGO_TILE, ALGO_SKINNY, ALGO_SMALL, ALGO_MFMA_ANY = -1, 0, 1, 2, 3, 4
 SCALE_TENSOR, SCALE_VECTOR = 0, 1
 OUT_F32, OUT_BF16 = 0, 1
 
@@ -66,6 +66,7 @@ SIGNATURES = {
     "cigemmDestroy": (_ci, [_vp]),
     "cigemmSetStream": (_ci, [_vp, _vp]),
     "cigemmGetStream": (_ci, [_vp, C.POINTER(_vp)]),
+    "cigemmResetWorkspace": (_ci, [_vp]),
     "cigemmGetStatusString": (C.c_char_p, [_ci]),
     "cigemmGetLastErrorString": (C.c_char_p, [_vp]),
     "cigemmGetVersion": (_ci, []),
@@ -74,9 +75,6 @@ SIGNATURES = {
     "cigemm_matrixMulTiled": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
     "cigemm_matrixMulMatrixCores": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
     "cigemm_matrixMulMatrixCoresBfloat16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int]),
-    "cigemm_probe_mfma": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int64)]),
-    "cigemm_probe_tile_phases": (C.c_int, [_vp, C.c_int, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp,
-                                           _i64, C.POINTER(C.c_double)]),
     "cigemmSetAlgo": (C.c_int, [_vp, C.c_int]),
     "cigemmGetAlgo": (C.c_int, [_vp, C.POINTER(C.c_int)]),
     "cigemm_gemm_f32": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
@@ -179,6 +177,10 @@ class Handle:
     def set_stream(self, raw_stream: int):
         self._check(self.lib.cigemmSetStream(self._h, _vp(raw_stream)), "cigemmSetStream")
 
+    def reset_workspace(self):
+        """Zero the split-K arrival counters and exchange words (after a failure seen elsewhere)."""
+        self._check(self.lib.cigemmResetWorkspace(self._h), "cigemmResetWorkspace")
+
     def set_algo(self, algo: int):
         """Restrict following GEMM calls to one kernel family (``ALGO_*``)."""
         self._check(self.lib.cigemmSetAlgo(self._h, algo), "cigemmSetAlgo")
@@ -261,31 +263,6 @@ class Handle:
         torch = _torch()
         assert A.dtype == torch.float16 and B.dtype == torch.float16
         return self._gemm("cigemm_gemm_f16", A, B, out, torch.float16)
-
-    def probe_mfma(self, kind: str, random_bits: bool, iters: int) -> int:
-        """Launch the register-resident matrix-core loop; returns the operations it performs."""
-        ops = C.c_int64(0)
-        k = {"bf16": 0, "f16": 1, "i8": 2, "bf16_16x16": 3, "f16_16x16": 4, "i8_16x16": 5,
-             "f32": 6}[kind]
-        self._check(self.lib.cigemm_probe_mfma(self._h, k, int(random_bits), iters, C.byref(ops)),
-                    "cigemm_probe_mfma")
-        return ops.value
-
-    def probe_tile_phases(self, A, B, out, paired=False):
-        """One instrumented launch of the 256-row tile kernel, or with ``paired`` of its
-        two-workgroups-per-unit form (bf16 or int8 K x N -> int32); returns the phase figures
-        as a dict (see cigemm_probe_tile_phases)."""
-        torch = _torch()
-        kind = {torch.bfloat16: 0, torch.int8: 1}[A.dtype] + (2 if paired else 0)
-        M, K = A.shape
-        N = B.shape[1]
-        ph = (C.c_double * 8)()
-        st = self.lib.cigemm_probe_tile_phases(self._h, kind, M, N, K, A.data_ptr(), self._ld(A),
-                                               B.data_ptr(), self._ld(B), out.data_ptr(), self._ld(out), ph)
-        self._check(st, "cigemm_probe_tile_phases")
-        keys = ("prologue_us", "main_loop_us", "epilogue_us", "first_start_to_last_end_us",
-                "cycles_per_stage", "main_loop_clock_ghz", "first_epilogue_to_last_end_us", "workgroups")
-        return dict(zip(keys, list(ph)))
 
     # -- study kernels (TileProgramming demo) -------------------------------------------------
     def matrixMulTiled(self, A, B):

@@ -1,70 +1,12 @@
 // C ABI: handle lifecycle, argument validation and dispatch to the kernel families.
 // Validation happens entirely on the host, before any launch: a call that returns a
 // non-success status has enqueued nothing.
-#include <cstdarg>
 #include <cstdlib>
 #include <new>
 
 #include "common.h"
 
 namespace cig {
-
-cigemmStatus_t fail(cigemmContext* ctx, cigemmStatus_t st, const char* fmt, ...) {
-  if (ctx) {
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(ctx->last_error, sizeof(ctx->last_error), fmt, ap);
-    va_end(ap);
-  }
-  return st;
-}
-
-cigemmStatus_t check_launch(cigemmContext* ctx, const char* what) {
-  if (ctx && ctx->pending_error[0]) {
-    char msg[sizeof(ctx->pending_error)];
-    memcpy(msg, ctx->pending_error, sizeof(msg));
-    ctx->pending_error[0] = '\0';
-    (void)hipGetLastError();
-    return fail(ctx, CIGEMM_STATUS_INTERNAL_ERROR, "%s: %s", what, msg);
-  }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess)
-    return fail(ctx, CIGEMM_STATUS_EXECUTION_FAILED, "%s: HIP error: %s", what,
-                hipGetErrorString(e));
-  return CIGEMM_STATUS_SUCCESS;
-}
-
-void set_tile_kernel_name(cigemmContext* ctx, const char* dtype, int k_elems, const char* suffix,
-                          bool splitk) {
-  char rows[24], waves[24];
-  if (ctx->first_tile_rows) {
-    snprintf(rows, sizeof(rows), "%d+%d", ctx->first_tile_rows, ctx->last_tile_rows);
-    snprintf(waves, sizeof(waves), "w%d+w%d", ctx->first_waves, ctx->last_waves);
-  } else {
-    snprintf(rows, sizeof(rows), "%d", ctx->last_tile_rows);
-    snprintf(waves, sizeof(waves), ctx->last_per_cu == 2 ? "w%dx2" : "w%d", ctx->last_waves);
-  }
-  snprintf(ctx->kernel_name, sizeof(ctx->kernel_name), "%s_mfma_%sx256x%d_%s_ring%d%s%s", dtype,
-           rows, k_elems, waves, ctx->last_per_cu == 2 ? 3 : 4, suffix, splitk ? "_splitk" : "");
-  ctx->last_kernel = ctx->kernel_name;
-}
-
-bool ensure_dynamic_lds(cigemmContext* ctx, const void* kernel, int bytes,
-                        std::atomic<uint64_t>& done) {
-  const uint64_t bit = 1ull << (ctx->device & 63);
-  if (done.load(std::memory_order_acquire) & bit) return true;
-  const hipError_t e =
-      hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-  if (e != hipSuccess) {
-    (void)hipGetLastError();
-    snprintf(ctx->pending_error, sizeof(ctx->pending_error),
-             "the device refused %d bytes of LDS per workgroup (%s)", bytes, hipGetErrorString(e));
-    return false;
-  }
-  done.fetch_or(bit, std::memory_order_release);
-  return true;
-}
-
 namespace {
 
 bool valid(cigemmHandle_t h) { return h && h->magic == kCtxMagic; }
@@ -79,6 +21,7 @@ cigemmStatus_t check_gemm_args(cigemmHandle_t h, const char* name, int64_t M, in
   h->last_per_cu = 1;
   h->first_tile_rows = 0;
   h->first_waves = 0;
+  if (h->ws_dirty) clear_workspace(h);  // a call before this one ended in EXECUTION_FAILED
   if (M < 0 || N < 0 || K < 0)
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: negative dimension (M=%lld N=%lld K=%lld)",
                 name, (long long)M, (long long)N, (long long)K);
@@ -145,6 +88,7 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->ws_partial_bytes = (size_t)64 << 20;
   ctx->ws_counter_bytes = (size_t)64 << 10;
   ctx->ws_swap_bytes = (size_t)8 << 20;  // 128 bytes per column: N <= 65536
+  ctx->ws_dirty = 0;
   ctx->workspace = nullptr;
   if (hipMalloc(&ctx->workspace,
                 ctx->ws_partial_bytes + ctx->ws_counter_bytes + ctx->ws_swap_bytes) != hipSuccess ||
@@ -171,6 +115,12 @@ cigemmStatus_t cigemmSetStream(cigemmHandle_t h, void* stream) {
   if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
   h->stream = static_cast<hipStream_t>(stream);
   return CIGEMM_STATUS_SUCCESS;
+}
+
+cigemmStatus_t cigemmResetWorkspace(cigemmHandle_t h) {
+  if (!valid(h)) return CIGEMM_STATUS_NOT_INITIALIZED;
+  clear_workspace(h);
+  return check_launch(h, "cigemmResetWorkspace");
 }
 
 cigemmStatus_t cigemmGetStream(cigemmHandle_t h, void** stream) {
@@ -243,7 +193,6 @@ static bool dispatch_f32(cigemmHandle_t h, int64_t M, int64_t N, int64_t K, cons
       launch_f32_small(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
       return true;
     case CIGEMM_ALGO_SKINNY:
-    case CIGEMM_ALGO_TILE_PAIRED:
       return false;
     case CIGEMM_ALGO_MFMA_ANY:
       return launch_mfma_any_f32(h, M, N, K, A, lda, B, ldb, C, ldc, ba);
@@ -292,9 +241,6 @@ static cigemmStatus_t gemm16(cigemmHandle_t h, const char* name, bool bf16, int6
   switch (h->algo) {
     case CIGEMM_ALGO_SKINNY: ok = launch_skinny_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
     case CIGEMM_ALGO_TILE: ok = launch_16b_mfma(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
-    case CIGEMM_ALGO_TILE_PAIRED:
-      ok = launch_16b_mfma_paired(h, bf16, M, N, K, A, lda, B, ldb, C, ldc);
-      break;
     case CIGEMM_ALGO_SMALL: ok = false; break;
     case CIGEMM_ALGO_MFMA_ANY: ok = launch_mfma_any_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
     case CIGEMM_ALGO_GENERIC: launch_generic_16(h, bf16, M, N, K, A, lda, B, ldb, C, ldc); break;
@@ -331,9 +277,6 @@ static cigemmStatus_t gemm_i8(cigemmHandle_t h, const char* name, int64_t M, int
   switch (h->algo) {
     case CIGEMM_ALGO_SKINNY: ok = launch_skinny_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq); break;
     case CIGEMM_ALGO_TILE: ok = launch_i8_mfma(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq); break;
-    case CIGEMM_ALGO_TILE_PAIRED:
-      ok = launch_i8_mfma_paired(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);
-      break;
     case CIGEMM_ALGO_SMALL: ok = false; break;
     case CIGEMM_ALGO_MFMA_ANY:
       ok = launch_mfma_any_i8(h, M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq);

@@ -35,6 +35,10 @@ struct cigemmContext {
   size_t ws_partial_bytes;
   size_t ws_counter_bytes;
   size_t ws_swap_bytes;
+  // Set when a call on this handle ended in CIGEMM_STATUS_EXECUTION_FAILED: a split-K kernel
+  // that did not run to its end may have left arrival counters or exchange words non-zero.
+  // The next GEMM call clears both (a small kernel on the handle's stream) before it launches.
+  int ws_dirty;
   char last_error[256];
 };
 
@@ -244,19 +248,14 @@ void launch_f32_small(cigemmContext*, int64_t M, int64_t N, int64_t K, const flo
 bool launch_16b_mfma(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
                      const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                      uint16_t* C, int64_t ldc);
-// The two-workgroups-per-unit form of the tile kernel (mfma_tile2.h), K x N operands only;
-// chosen only by cigemmSetAlgo(CIGEMM_ALGO_TILE_PAIRED).
-bool launch_16b_mfma_paired(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
-                            const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
-                            uint16_t* C, int64_t ldc);
-bool launch_i8_mfma_paired(cigemmContext*, int64_t M, int64_t N, int64_t K, const int8_t* A,
-                           int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
-                           int64_t ldc, const DequantArgs* dq);
 // gemm_i8.hip
 bool launch_i8_mfma(cigemmContext*, int64_t M, int64_t N, int64_t K, const int8_t* A,
                     int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
                     int64_t ldc, const DequantArgs* dq);
 // gemm_skinny.hip
+// Enqueues a kernel on the handle's stream that zeroes the arrival counters and the exchange
+// words of the handle's workspace, and takes the dirty mark off the handle.
+void clear_workspace(cigemmContext*);
 bool launch_skinny_16(cigemmContext*, bool bf16, int64_t M, int64_t N, int64_t K,
                       const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
                       uint16_t* C, int64_t ldc);

@@ -3,7 +3,7 @@
 // out.  The kernel itself is the shared LDS-tiled MFMA kernel; this file supplies the
 // 16-bit epilogue and the shape gate.
 #include "epilogues.h"
-#include "mfma_tile2.h"
+#include "mfma_tile.h"
 
 namespace cig {
 
@@ -21,21 +21,6 @@ bool launch_16b_mfma(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_
         ctx, M, N, K * 2, A, lda * 2, B, ldb * 2, EpiStore16x4<F16>{C, ldc});
     set_tile_kernel_name(ctx, "f16", 32, "", split);
   }
-  return true;
-}
-
-bool launch_16b_mfma_paired(cigemmContext* ctx, bool bf16, int64_t M, int64_t N, int64_t K,
-                            const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
-                            uint16_t* C, int64_t ldc) {
-  if (!tile::tile_shape_ok(M, N, K, 2, A, lda, B, ldb, true)) return false;
-  if (ldc % 8 || ((uintptr_t)C & 15)) return false;
-  if (bf16)
-    tile::launch_tile2<tile::MathBF16, tile::B_KN16>(ctx, M, N, K * 2, A, lda * 2, B, ldb * 2,
-                                                     EpiStore16x4<BF16>{C, ldc});
-  else
-    tile::launch_tile2<tile::MathF16, tile::B_KN16>(ctx, M, N, K * 2, A, lda * 2, B, ldb * 2,
-                                                    EpiStore16x4<F16>{C, ldc});
-  set_tile_kernel_name(ctx, bf16 ? "bf16" : "f16", 32, "", false);
   return true;
 }
 

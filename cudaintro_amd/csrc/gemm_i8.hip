@@ -2,32 +2,10 @@
 // with either raw int32 output or the fused scale-and-dequantize epilogue.  The kernel is
 // the shared LDS-tiled MFMA kernel; this file supplies the int8 epilogues and the gate.
 #include "epilogues.h"
-#include "mfma_tile2.h"
+#include "mfma_tile.h"
 
 namespace cig {
 namespace {
-
-// The two-workgroups-per-unit form (K x N operands).
-void launch_kn_tile2(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
-                     int64_t lda, const int8_t* B, int64_t ldb, int32_t* C, int64_t ldc,
-                     const DequantArgs* dq) {
-  if (!dq) {
-    tile::launch_tile2<tile::MathI8, tile::B_KN8>(ctx, M, N, K, A, lda, B, ldb, EpiStoreI32x4{C, ldc});
-    return;
-  }
-#define CIG_DQ2(OB, DA)                                                                       \
-  tile::launch_tile2<tile::MathI8, tile::B_KN8>(                                              \
-      ctx, M, N, K, A, lda, B, ldb,                                                           \
-      EpiDequantX4<OB, DA>{dq->out, dq->ldo, dq->sa, dq->sb, dq->sa_vec, dq->sb_vec,          \
-                           dq->acc_out, dq->ldacc})
-  const bool dump = dq->acc_out != nullptr;
-  if (dq->out_bf16) {
-    if (dump) CIG_DQ2(true, true); else CIG_DQ2(true, false);
-  } else {
-    if (dump) CIG_DQ2(false, true); else CIG_DQ2(false, false);
-  }
-#undef CIG_DQ2
-}
 
 template <int BMODE>
 bool launch_layout(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
@@ -53,34 +31,10 @@ bool launch_layout(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const in
 
 }  // namespace
 
-static bool i8_tile_ok(int64_t M, int64_t N, int64_t K, const int8_t* A, int64_t lda,
-                       const int8_t* B, int64_t ldb, bool b_nk, const int32_t* C, int64_t ldc,
-                       const DequantArgs* dq) {
-  if (!tile::tile_shape_ok(M, N, K, 1, A, lda, B, ldb, !b_nk)) return false;
-  if (!dq) {
-    if (ldc % 4 || ((uintptr_t)C & 15)) return false;
-  } else {
-    if (dq->ldo % (dq->out_bf16 ? 8 : 4) || ((uintptr_t)dq->out & 15))
-      return false;  // output rows are stored in 16-byte pieces
-    if (dq->sb_vec && ((uintptr_t)dq->sb & 15)) return false;
-    if (dq->acc_out && (dq->ldacc % 4 || ((uintptr_t)dq->acc_out & 15))) return false;
-  }
-  return true;
-}
-
-bool launch_i8_mfma_paired(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
-                           int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C,
-                           int64_t ldc, const DequantArgs* dq) {
-  if (b_nk || !i8_tile_ok(M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq)) return false;
-  launch_kn_tile2(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
-  set_tile_kernel_name(ctx, "i8", 64, dq ? "_kn_dequant" : "_kn", false);
-  return true;
-}
-
 bool launch_i8_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const int8_t* A,
                     int64_t lda, const int8_t* B, int64_t ldb, bool b_nk, int32_t* C, int64_t ldc,
                     const DequantArgs* dq) {
-  if (!i8_tile_ok(M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq)) return false;
+  if (!tile::i8_tile_ok(M, N, K, A, lda, B, ldb, b_nk, C, ldc, dq)) return false;
   const bool split = b_nk ? launch_layout<tile::B_NK>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq)
                           : launch_layout<tile::B_KN8>(ctx, M, N, K, A, lda, B, ldb, C, ldc, dq);
   set_tile_kernel_name(ctx, "i8", 64, dq ? (b_nk ? "_nk_dequant" : "_kn_dequant") : (b_nk ? "_nk" : "_kn"),

@@ -404,17 +404,11 @@ __global__ __launch_bounds__(256, 1) void skinny_kernel(int M, int N, int stages
   if (t == 0) __hip_atomic_store(counters + slab, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Number of K splits, a power of two up to 16: enough workgroups to cover the chip about
-// once, at least 4 stages per split, and partials that fit the workspace.
+// Number of K splits: skinny_plan.h has the rule.
 template <typename Geo>
 int choose_splits(const cigemmContext* ctx, int64_t N, int64_t kts) {
-  const int64_t slabs = N / Geo::BN;
-  int s = 1;
-  while (s < 16 && slabs * s < ctx->num_cus && kts % (2 * s) == 0 && kts / (2 * s) >= 4 &&
-         (size_t)(2 * s) * XROWS * N * 4 <= ctx->ws_partial_bytes)
-    s *= 2;
-  if ((size_t)slabs * 4 > ctx->ws_counter_bytes) s = 1;
-  return s;
+  return skinny_plan::barrier_kernel_splits(N / Geo::BN, N, kts, XROWS, ctx->num_cus,
+                                            ctx->ws_counter_bytes, ctx->ws_partial_bytes);
 }
 
 template <typename Geo, typename Epi, int SPLITS>
@@ -1261,6 +1255,23 @@ __global__ void clear_counters_kernel(uint32_t* counters, int n, uint64_t* swap_
   if (i < n) counters[i] = 0;
   for (int64_t j = i; j < n_swap_words; j += (int64_t)gridDim.x * blockDim.x) swap_words[j] = 0;
 }
+
+}  // namespace
+
+void clear_workspace(cigemmContext* ctx) {
+  ctx->ws_dirty = 0;
+  if (!ctx->workspace) return;
+  char* base = static_cast<char*>(ctx->workspace) + ctx->ws_partial_bytes;
+  const int counters = (int)(ctx->ws_counter_bytes / 4);
+  const int64_t words = (int64_t)(ctx->ws_swap_bytes / 8);
+  const int blocks = 4 * (ctx->num_cus > 0 ? ctx->num_cus : 256);
+  const int need = (counters + 255) / 256;
+  hipLaunchKernelGGL(clear_counters_kernel, dim3(blocks > need ? blocks : need), dim3(256), 0,
+                     ctx->stream, reinterpret_cast<uint32_t*>(base), counters,
+                     reinterpret_cast<uint64_t*>(base + ctx->ws_counter_bytes), words);
+}
+
+namespace {
 
 cigemmStatus_t static_fail(char* err, size_t err_len, cigemmStatus_t st, const char* fmt, ...)
     __attribute__((format(printf, 4, 5)));

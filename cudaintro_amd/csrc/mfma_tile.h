@@ -1142,5 +1142,21 @@ inline bool tile_shape_ok(int64_t M, int64_t N, int64_t K, int elem, const void*
   return true;
 }
 
+// The int8 tile kernels' gate: the shape gate above plus what their epilogues store in 16-byte
+// pieces (output rows, the accumulator dump) or load as such (per-column scales).
+inline bool i8_tile_ok(int64_t M, int64_t N, int64_t K, const int8_t* A, int64_t lda,
+                       const int8_t* B, int64_t ldb, bool b_nk, const int32_t* C, int64_t ldc,
+                       const DequantArgs* dq) {
+  if (!tile_shape_ok(M, N, K, 1, A, lda, B, ldb, !b_nk)) return false;
+  if (!dq) {
+    if (ldc % 4 || ((uintptr_t)C & 15)) return false;
+  } else {
+    if (dq->ldo % (dq->out_bf16 ? 8 : 4) || ((uintptr_t)dq->out & 15)) return false;
+    if (dq->sb_vec && ((uintptr_t)dq->sb & 15)) return false;
+    if (dq->acc_out && (dq->ldacc % 4 || ((uintptr_t)dq->acc_out & 15))) return false;
+  }
+  return true;
+}
+
 }  // namespace tile
 }  // namespace cig

@@ -2,6 +2,10 @@
 // wave per SIMD on every compute unit, to show what the chip sustains at the clock it
 // actually holds under this load.  Sustained rate depends on the operand data (the chip is
 // power limited), so the probe runs on constant or on pseudo-random operand bits.
+#include <algorithm>
+#include <vector>
+
+#include "cigemm_probe.h"
 #include "common.h"
 
 namespace cig {
@@ -97,6 +101,140 @@ __global__ __launch_bounds__(256, 1) void mfma_probe_kernel(float* __restrict__ 
   out[blockIdx.x * 256 + threadIdx.x] = s;
 }
 
+
+// ---- what the other instructions of the tile kernel's main loop cost ---------------------
+// One "stage" = two k-steps of 16 bf16 32x32x16 matrix instructions on a 4 x 4 grid of
+// accumulator tiles (the 128 x 128 wave tile of the product kernel), fragments double buffered
+// in registers.  Optional, at the places the product kernel's schedule puts them: 12 LDS
+// fragment reads per k-step (4 of 16 bytes, 8 transposing ones of 8 bytes) for the other
+// fragment buffer, NDMA LDS-DMA instructions in the second k-step, one wait and one workgroup
+// barrier between the k-steps.  Every slot (one matrix instruction, at most one read, at most
+// one DMA) is closed by a scheduling fence.
+typedef __attribute__((address_space(3))) i16x4 probe_lds_i16x4;
+
+template <int NDMA, int NLDS, int BARRIER>
+__global__ __launch_bounds__(256, 1) void issue_cost_kernel(const char* __restrict__ src,
+                                                            uint64_t* __restrict__ stamps,
+                                                            float* __restrict__ sink, int iters) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int t = threadIdx.x, l = t & 63;
+  const int w = __builtin_amdgcn_readfirstlane(t >> 6);
+  // per wave: 8 KiB that the fragment reads read, 8 KiB that the DMA fills and nothing reads
+  char* rd = lds + w * 16384;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  const uint32_t dma_dst = lds_base + w * 16384 + 8192;
+  for (int i = l * 16; i < 8192; i += 1024) {
+    u32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)  // +-[1,2) in bf16, pseudo-random sign and mantissa
+      v[e] = (mix32((uint32_t)(blockIdx.x * 65536 + w * 8192 + i + e + 1)) & 0x807f807fu) | 0x3f803f80u;
+    *reinterpret_cast<u32x4*>(rd + i) = v;
+  }
+  __syncthreads();
+  const char* my_src = src + ((size_t)blockIdx.x * 4 + w) * 8192;
+  const uint32_t voff = (uint32_t)l * 16;
+  struct Frags {
+    u32x4 a[4];
+    u32x2 b[8];
+  };
+  auto read_piece = [&](Frags& f, int kk, int r) {
+    if (r < 4)
+      f.a[r] = *reinterpret_cast<const u32x4*>(rd + (r ^ kk) * 1024 + l * 16);
+    else
+      f.b[r - 4] = __builtin_bit_cast(
+          u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                     (probe_lds_i16x4*)(rd + 4096 + ((r - 4) ^ kk) * 512 + l * 8)));
+  };
+  Frags f0, f1;
+#pragma unroll
+  for (int r = 0; r < 12; ++r) read_piece(f0, 0, r);
+#pragma unroll
+  for (int r = 0; r < 12; ++r) read_piece(f1, 1, r);
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  auto mfma_piece = [&](const Frags& f, int m) {
+    const int j = m / 4;
+    const int i = (j & 1) ? 3 - m % 4 : m % 4;
+    const u32x4 bfrag = __builtin_shufflevector(f.b[2 * j], f.b[2 * j + 1], 0, 1, 2, 3);
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bfrag),
+                                                        __builtin_bit_cast(bf16x8, f.a[i]),
+                                                        acc[i][j], 0, 0, 0);
+  };
+  uint64_t t0 = 0, r0 = 0;
+  if (l == 0) {
+    t0 = __builtin_amdgcn_s_memtime();
+    r0 = __builtin_amdgcn_s_memrealtime();
+  }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int sl = 0; sl < 16; ++sl) {
+      mfma_piece(f0, sl);
+      if (NLDS && sl < 12) read_piece(f1, 1, sl);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // (as in the product: everything but the DMA of the last two stages has landed)
+    if (NDMA) __builtin_amdgcn_s_waitcnt(0x0f70 | ((2 * NDMA) & 15) | (((2 * NDMA) >> 4) << 14));
+    if (BARRIER) __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int sl = 0; sl < 16; ++sl) {
+      mfma_piece(f1, sl);
+      if (NLDS && sl < 12) read_piece(f0, 0, sl);
+      if (sl < NDMA)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(dma_dst + sl * 1024), "v"(voff), "s"(my_src)
+                     : "m0");
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("" ::: "memory");
+  }
+  if (l == 0) {
+    uint64_t* p = stamps + ((size_t)blockIdx.x * 4 + w) * 4;
+    p[0] = t0;
+    p[1] = __builtin_amdgcn_s_memtime();
+    p[2] = r0;
+    p[3] = __builtin_amdgcn_s_memrealtime();
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): no DMA outlives the wave
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sum += acc[i][j][e];
+  sink[blockIdx.x * 256 + t] = sum;
+}
+
+// Microseconds per tick of the constant-rate counter s_memrealtime reads.
+double wall_tick_us(int device) {
+  int khz = 0;
+  if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) != hipSuccess || khz <= 0) {
+    (void)hipGetLastError();
+    return 0.01;  // 100 MHz, gfx950's rate
+  }
+  return 1.0e3 / (double)khz;
+}
+
+constexpr int ISSUE_LDS_BYTES = 4 * 16384;
+
+template <int NDMA, int NLDS, int BARRIER>
+void launch_issue_cost(cigemmContext* ctx, int grid, const char* src, uint64_t* stamps, float* sink,
+                       int iters) {
+  auto kern = issue_cost_kernel<NDMA, NLDS, BARRIER>;
+  static std::atomic<uint64_t> lds_set{0};
+  if (!ensure_dynamic_lds(ctx, (const void*)kern, ISSUE_LDS_BYTES, lds_set)) return;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), ISSUE_LDS_BYTES, ctx->stream, src, stamps, sink,
+                     iters);
+}
+
 }  // namespace
 }  // namespace cig
 
@@ -130,4 +268,89 @@ extern "C" cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t h, int kind, int rand
                       (kind == 2 ? 65536 : kind == 6 ? 4096 : kind == 5 ? 32768 : kind >= 3 ? 16384 : 32768);
   h->last_kernel = "mfma_probe";
   return check_launch(h, "cigemm_probe_mfma");
+}
+
+extern "C" cigemmStatus_t cigemm_probe_issue_cost(cigemmHandle_t h, int n_dma, int n_lds_reads,
+                                                  int barrier, int workgroups, int iters,
+                                                  double* result) {
+  const char* name = "cigemm_probe_issue_cost";
+  if (!h || h->magic != kCtxMagic) return CIGEMM_STATUS_NOT_INITIALIZED;
+  const int cus = h->num_cus > 0 ? h->num_cus : 256;
+  if ((n_dma != 0 && n_dma != 2 && n_dma != 4 && n_dma != 8) ||
+      (n_lds_reads != 0 && n_lds_reads != 24) || (barrier != 0 && barrier != 1) || workgroups < 1 ||
+      workgroups > cus || iters <= 0 || iters > (1 << 22) || !result)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE,
+                "%s: n_dma %d (0, 2, 4, 8), n_lds_reads %d (0, 24), barrier %d, workgroups %d "
+                "(1..%d), iters %d", name, n_dma, n_lds_reads, barrier, workgroups, cus, iters);
+  // workspace: stamps (32 bytes per wave), the sink, then 8 KiB of DMA source per wave
+  const size_t stamp_bytes = (size_t)workgroups * 4 * 32, sink_bytes = (size_t)workgroups * 1024;
+  const size_t src_off = (stamp_bytes + sink_bytes + 4095) & ~(size_t)4095;
+  if (!h->workspace || src_off + (size_t)workgroups * 4 * 8192 > h->ws_partial_bytes)
+    return fail(h, CIGEMM_STATUS_ALLOC_FAILED, "%s: workspace too small", name);
+  char* ws = static_cast<char*>(h->workspace);
+  uint64_t* stamps = reinterpret_cast<uint64_t*>(ws);
+  float* sink = reinterpret_cast<float*>(ws + stamp_bytes);
+  const char* src = ws + src_off;
+#define CIG_IC(D, L, B) launch_issue_cost<D, L, B>(h, workgroups, src, stamps, sink, iters)
+#define CIG_IC_B(D, L) do { if (barrier) CIG_IC(D, L, 1); else CIG_IC(D, L, 0); } while (0)
+#define CIG_IC_L(D) do { if (n_lds_reads) CIG_IC_B(D, 24); else CIG_IC_B(D, 0); } while (0)
+  switch (n_dma) {
+    case 0: CIG_IC_L(0); break;
+    case 2: CIG_IC_L(2); break;
+    case 4: CIG_IC_L(4); break;
+    default: CIG_IC_L(8); break;
+  }
+#undef CIG_IC_L
+#undef CIG_IC_B
+#undef CIG_IC
+  cigemmStatus_t st = check_launch(h, name);
+  if (st != CIGEMM_STATUS_SUCCESS) return st;
+  std::vector<uint64_t> host((size_t)workgroups * 16);
+  if (hipMemcpyAsync(host.data(), stamps, host.size() * 8, hipMemcpyDeviceToHost, h->stream) != hipSuccess ||
+      hipStreamSynchronize(h->stream) != hipSuccess) {
+    (void)hipGetLastError();
+    h->ws_dirty = 1;
+    return fail(h, CIGEMM_STATUS_EXECUTION_FAILED, "%s: reading the stamps back failed", name);
+  }
+  const double tick_us = wall_tick_us(h->device);
+  double cycles = 0, worst = 0, ticks = 0;
+  uint64_t first = ~0ull, last = 0;
+  for (int i = 0; i < workgroups * 4; ++i) {
+    const uint64_t* p = &host[(size_t)i * 4];
+    const double c = (double)(p[1] - p[0]);
+    cycles += c;
+    worst = std::max(worst, c);
+    ticks += (double)(p[3] - p[2]);
+    first = std::min(first, p[2]);
+    last = std::max(last, p[3]);
+  }
+  result[0] = cycles / (workgroups * 4) / iters;
+  result[1] = worst / iters;
+  result[2] = ticks > 0 ? cycles / (ticks * tick_us) * 1e-3 : 0.0;
+  result[3] = (double)(last - first) * tick_us;
+  h->last_kernel = "issue_cost_probe";
+  return CIGEMM_STATUS_SUCCESS;
+}
+
+extern "C" cigemmStatus_t cigemm_probe_dirty_workspace(cigemmHandle_t h, int count, uint32_t value,
+                                                       int mark_dirty) {
+  const char* name = "cigemm_probe_dirty_workspace";
+  if (!h || h->magic != kCtxMagic) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if (count < 0 || (size_t)count * 4 > h->ws_counter_bytes || (size_t)count * 8 > h->ws_swap_bytes ||
+      !h->workspace)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: count %d", name, count);
+  if (count > 0) {
+    char* base = static_cast<char*>(h->workspace) + h->ws_partial_bytes;
+    std::vector<uint32_t> c32((size_t)count, value);
+    std::vector<uint64_t> c64((size_t)count, ((uint64_t)value << 32) | value);
+    if (hipMemcpyAsync(base, c32.data(), c32.size() * 4, hipMemcpyHostToDevice, h->stream) != hipSuccess ||
+        hipMemcpyAsync(base + h->ws_counter_bytes, c64.data(), c64.size() * 8, hipMemcpyHostToDevice,
+                       h->stream) != hipSuccess ||
+        hipStreamSynchronize(h->stream) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(h, CIGEMM_STATUS_EXECUTION_FAILED, "%s: copy failed", name);
+    }
+  }
+  if (mark_dirty) h->ws_dirty = 1;
+  return CIGEMM_STATUS_SUCCESS;
 }

@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <vector>
 
+#include "cigemm_probe.h"
 #include "epilogues.h"
 #include "mfma_tile2.h"
 
@@ -35,10 +36,18 @@ cigemmStatus_t run_profiled(cigemmContext* ctx, const char* name, int64_t M, int
   if (hipMemcpyAsync(h.data(), stamps, h.size() * 8, hipMemcpyDeviceToHost, ctx->stream) != hipSuccess ||
       hipStreamSynchronize(ctx->stream) != hipSuccess) {
     (void)hipGetLastError();
+    ctx->ws_dirty = 1;
     return fail(ctx, CIGEMM_STATUS_EXECUTION_FAILED, "%s: reading the stamps back failed", name);
   }
-  // constant-rate counter: 100 MHz on this chip (10 ns per tick)
-  const double tick_us = 0.01;
+  // microseconds per tick of the constant-rate counter (100 MHz on gfx950)
+  double tick_us = 0.01;
+  {
+    int khz = 0;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, ctx->device) == hipSuccess && khz > 0)
+      tick_us = 1.0e3 / (double)khz;
+    else
+      (void)hipGetLastError();
+  }
   const int64_t kts = (K_bytes + tile::KB - 1) / tile::KB;
   double phase_us[3] = {0, 0, 0}, main_cycles = 0, main_ticks = 0;
   uint64_t first_start = ~0ull, last_end = 0, first_epi = ~0ull, last_main_end = 0;
@@ -57,7 +66,8 @@ cigemmStatus_t run_profiled(cigemmContext* ctx, const char* name, int64_t M, int
   out[2] = phase_us[2] / tiles;                       // epilogue, stores acknowledged
   out[3] = (double)(last_end - first_start) * tick_us;  // first workgroup start -> last end
   out[4] = main_cycles / tiles / (double)kts;         // shader cycles per 64-byte stage
-  out[5] = main_cycles / (main_ticks * tick_us) * 1e-3;  // GHz held in the main loop
+  // GHz held in the main loop (0 when it is shorter than a tick of the wall clock)
+  out[5] = main_ticks > 0 ? main_cycles / (main_ticks * tick_us) * 1e-3 : 0.0;
   out[6] = (double)(last_end - first_epi) * tick_us;  // first epilogue start -> last end
   out[7] = (double)tiles;
   ctx->last_kernel = "tile_phase_probe";
@@ -75,17 +85,21 @@ extern "C" cigemmStatus_t cigemm_probe_tile_phases(cigemmHandle_t h, int kind, i
                                                    void* C, int64_t ldc, double* phases) {
   const char* name = "cigemm_probe_tile_phases";
   if (!h || h->magic != kCtxMagic) return CIGEMM_STATUS_NOT_INITIALIZED;
-  if (kind < 0 || kind > 3 || !A || !B || !C || !phases || M <= 0 || N <= 0 || K <= 0 ||
+  if (kind < 0 || kind > 4 || !A || !B || !C || !phases || M <= 0 || N <= 0 || K <= 0 ||
       lda < K || ldb < N || ldc < N)
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: bad argument", name);
-  const int elem = (kind & 1) == 0 ? 2 : 1;
+  const int elem = (kind == 1 || kind == 3) ? 1 : 2;
   if (!tile::tile_shape_ok(M, N, K, elem, A, lda, B, ldb, true) || N % 8 || ldc % 8 ||
       ((uintptr_t)C & 15))
     return fail(h, CIGEMM_STATUS_NOT_SUPPORTED, "%s: shape or alignment outside the tile kernel's",
                 name);
   const EpiStore16x4<BF16> e16{static_cast<uint16_t*>(C), ldc};
   const EpiStoreI32x4 e32{static_cast<int32_t*>(C), ldc};
+  const EpiStore16x4<F16> e16h{static_cast<uint16_t*>(C), ldc};
   switch (kind) {
+    case 4:
+      return run_profiled<tile::MathF16, tile::B_KN16, false>(h, name, M, N, K * 2, A, lda * 2, B,
+                                                              ldb * 2, e16h, phases);
     case 0:
       return run_profiled<tile::MathBF16, tile::B_KN16, false>(h, name, M, N, K * 2, A, lda * 2, B,
                                                                ldb * 2, e16, phases);

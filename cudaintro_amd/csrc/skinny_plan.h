@@ -34,6 +34,20 @@ inline int kwaves_splits(int64_t slabs, int64_t stages, int cols, int cus, size_
   return best;
 }
 
+// The kernel with 256-column (16-bit) or 128-column (int8) slabs and a workgroup barrier per
+// stage: number of K ranges, a power of two up to 16 -- enough workgroups to cover the chip
+// about once, at least 4 stages per range, partials (`xrows` rows of 4-byte sums per column and
+// range) and counters within the workspace.
+inline int barrier_kernel_splits(int64_t slabs, int64_t N, int64_t stages, int xrows, int cus,
+                                 size_t counter_bytes, size_t partial_bytes) {
+  int s = 1;
+  while (s < 16 && slabs * s < cus && stages % (2 * s) == 0 && stages / (2 * s) >= 4 &&
+         (size_t)(2 * s) * (size_t)xrows * (size_t)N * 4 <= partial_bytes)
+    s *= 2;
+  if ((size_t)slabs * 4 > counter_bytes) s = 1;
+  return s;
+}
+
 // int8 N x K weights in 32-row slabs, few slabs and more than `xr` rows of x: the rows are cut into
 // tiles of `xr` rows (8 or 16) that get workgroups of their own, as long as every workgroup
 // still finds a compute unit and the slabs come in whole groups of 8 (the block order then

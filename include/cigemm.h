@@ -17,6 +17,15 @@
  *     return without synchronising (like cublasGemmEx).  Nothing is allocated per call.
  *   - Errors come back as codes; the library never exits the process.  The message of
  *     the last failing call on a handle is kept in cigemmGetLastErrorString().
+ *   - Operand rows are fetched in aligned 16-byte pieces wherever the rows are 16-byte aligned
+ *     (pointer and leading dimension): when a row's last piece is only partly inside the matrix
+ *     (16-bit N % 8 != 0, int8 N % 16 != 0 for K x N operands) the piece is still read whole.
+ *     For every row but the last that is row padding or the next row; for the LAST row of a
+ *     K x N operand it is up to 12 bytes past the (K-1)*ldb + N elements cublasGemmEx's
+ *     convention requires.  An aligned 16-byte piece never crosses a page, so this cannot
+ *     fault, and what is read there only feeds columns that are never stored; but the bytes up
+ *     to the next 16-byte boundary after the last element must be readable memory of the same
+ *     allocation granule (any allocator that hands out 16-byte multiples satisfies this).
  *   - A handle is not thread-safe; use one per host thread.
  *   - There is no CPU fallback: without a gfx950 device cigemmCreate() fails.
  */
@@ -85,9 +94,20 @@ CIGEMM_API cigemmStatus_t cigemmDestroy(cigemmHandle_t handle);
  * enqueued on the old one may still be running, or replaying a captured graph concurrently
  * with eager calls on the same handle, races on that workspace and gives wrong results
  * without an error.  Order the streams yourself (an event) before switching, or use one
- * handle per stream. */
+ * handle per stream.  (A kernel cut short mid-call: see cigemmResetWorkspace.) */
 CIGEMM_API cigemmStatus_t cigemmSetStream(cigemmHandle_t handle, void* stream);
 CIGEMM_API cigemmStatus_t cigemmGetStream(cigemmHandle_t handle, void** stream);
+
+/* Puts the handle's workspace back into the state cigemmCreate left it in: enqueues, on the
+ * handle's stream, a small kernel that zeroes the split-K arrival counters and exchange words.
+ * The library does this by itself before the next GEMM after a call on the handle returned
+ * CIGEMM_STATUS_EXECUTION_FAILED.  Call it when the failure was seen elsewhere: a kernel of
+ * this library that was aborted mid-run (a device reset, a stream destroyed under it) and
+ * reported by a later HIP call of the caller's own may have left a counter non-zero, and
+ * split-K shapes would then give wrong results without an error.  No counterpart in the
+ * reference (cuBLAS keeps no state between quantization/GEMM_*.cu's calls that a failed call
+ * could spoil). */
+CIGEMM_API cigemmStatus_t cigemmResetWorkspace(cigemmHandle_t handle);
 
 /* Replaces cublas_status_to_string (quantization/gemm_common.h:10-35). */
 CIGEMM_API const char* cigemmGetStatusString(cigemmStatus_t status);
@@ -127,12 +147,7 @@ typedef enum cigemmAlgo {
                               K x N); M <= 64 for K x N weights of at least 4096 x 2048 in
                               whole 128-column slabs */
   CIGEMM_ALGO_SMALL = 3,   /* fp32 32x32 tile per workgroup, k split over the waves */
-  CIGEMM_ALGO_TILE_PAIRED = 4, /* LDS-tiled MFMA kernel with 128-row tiles, two workgroups resident
-                              per compute unit and out of phase (16-bit, int8 K x N).  Never
-                              chosen by DEFAULT: it issues more matrix instructions per cycle and
-                              is slower on a power-limited chip; kept selectable as the measured
-                              counterpart of CIGEMM_ALGO_TILE */
-  CIGEMM_ALGO_MFMA_ANY = 5 /* 128x128 MFMA tiles fed by bounds-checked loads and stores at element
+  CIGEMM_ALGO_MFMA_ANY = 4 /* 128x128 MFMA tiles fed by bounds-checked loads and stores at element
                               alignment: any shape, leading dimension and alignment, every type.
                               DEFAULT uses it for what the families above do not take */
 } cigemmAlgo_t;
@@ -190,7 +205,8 @@ CIGEMM_API cigemmStatus_t cigemm_gemm_i8_dequant(
  * cigemm_gemm_bf16 on the same arguments; the kernel's scratch memory (split-K partial sums,
  * arrival counters and exchange words) is a fixed device array of 18 MiB + 4 KiB inside the library, which
  * every GPU the process uses holds until the process ends.
- *   Limits: 1 <= M <= 32, N <= 16384, N % 256 == 0, K % 32 == 0, lda and ldb multiples of 8,
+ *   Limits: 1 <= M <= 32, N <= 16384, N % 256 == 0, K >= 32 and K % 32 == 0 (K = 0, which
+ *   cigemm_gemm_bf16 answers with zeros, is refused here), lda and ldb multiples of 8,
  *   ldc a multiple of 4, A and B 16-byte aligned, C 8-byte aligned; anything else returns
  *   CIGEMM_STATUS_NOT_SUPPORTED (CIGEMM_STATUS_INVALID_VALUE for null pointers, negative sizes
  *   or leading dimensions below the row length) and launches nothing.
@@ -241,36 +257,6 @@ CIGEMM_API cigemmStatus_t cigemm_matrixMulMatrixCoresBfloat16(cigemmHandle_t han
                                                               const uint16_t* A,
                                                               const uint16_t* B, float* C,
                                                               int width);
-
-/* ---- measurement aid ------------------------------------------------------------------ */
-
-/* No counterpart in the reference.  Launches a register-resident matrix-core loop (no memory
- * traffic inside the loop) on every compute unit of the handle's device, on the handle's
- * stream: kind 0 = bf16 32x32x16, 1 = fp16 32x32x16, 2 = int8 32x32x32, 3 = bf16 16x16x32,
- * 4 = fp16 16x16x32, 5 = int8 16x16x64, 6 = fp32 32x32x2; random_bits 0 =
- * constant operands, 1 = pseudo-random operand bits (sustained clocks depend on the data);
- * `iters` loop trips of 12 instructions per wave.  *ops_per_launch receives 2.M.N.K summed
- * over all instructions, for the caller to divide by the time it measures. */
-CIGEMM_API cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t handle, int kind, int random_bits,
-                                            int iters, int64_t* ops_per_launch);
-
-/* No counterpart in the reference.  Runs ONE launch of the 256-row, four-wave LDS-tiled
- * matrix-core kernel (the product kernel with four timestamps added per workgroup) on the
- * handle's stream, waits for it, and reduces the stamps: kind 0 = bf16 (A, B, C as in
- * cigemm_gemm_bf16), 1 = int8 K x N operands, int32 out (as cigemm_gemm_i8_i32 with
- * CIGEMM_B_KN); 2 and 3 = the same two on the CIGEMM_ALGO_TILE_PAIRED form of the kernel
- * (128-row tiles; "stage" then means a stage of such a tile, 512 matrix-core issue cycles
- * instead of 1024).  Same shape and alignment conditions as the tile kernel, N % 8 == 0.
- * phases[0..7] receive, averaged over the workgroups: microseconds from workgroup start to the
- * first stage in registers; of the main loop; of the epilogue until its stores are
- * acknowledged; microseconds from the first workgroup's start to the last one's end; shader
- * cycles per 64-byte stage of k in the main loop; shader clock (GHz) held in the main loop;
- * microseconds from the first workgroup entering its epilogue to the last one's end; number of
- * workgroups.  Synchronises the stream; meant for profiling runs, not for the hot path. */
-CIGEMM_API cigemmStatus_t cigemm_probe_tile_phases(cigemmHandle_t handle, int kind, int64_t M,
-                                                   int64_t N, int64_t K, const void* A,
-                                                   int64_t lda, const void* B, int64_t ldb,
-                                                   void* C, int64_t ldc, double* phases);
 
 /* ---- device-side input generation -------------------------------------------------- */
 

@@ -6,6 +6,7 @@
 
 #include "skinny_plan.h"
 
+using cig::skinny_plan::barrier_kernel_splits;
 using cig::skinny_plan::kwaves_splits;
 using cig::skinny_plan::nk8_row_tiles;
 using cig::skinny_plan::two_tiles_fit;
@@ -85,6 +86,28 @@ int main() {
           }
           if (failures > 20) return 1;
         }
+  // The entry point that allocates nothing plans with a 16 MiB partial area and 4 KiB of
+  // counters where a handle has 64 MiB and 64 KiB, and promises the same bits as the handle
+  // entry: up to its limit of N = 16384 both must pick the same K ranges, in every kernel it
+  // can dispatch to (64- and 128-column slabs of the K-over-the-waves kernel, two row tiles
+  // included, and the 256-column slabs of the barrier kernel), for every K.
+  for (int64_t N = 64; N <= 16384; N += 64)
+    for (int64_t K = 32; K <= 32768; K += (K < 4096 ? 32 : 416)) {
+      const size_t sc = 4096, sp = (size_t)16 << 20, hc = (size_t)64 << 10, hp = (size_t)64 << 20;
+      for (int cols : {64, 128})
+        if (N % cols == 0 && K % 64 == 0)
+          for (int x_tiles : {1, 2}) {
+            ++checked;
+            EXPECT(kwaves_splits(N / cols, K / 64, cols, 256, sc, sp / x_tiles) ==
+                   kwaves_splits(N / cols, K / 64, cols, 256, hc, hp / x_tiles));
+          }
+      if (N % 256 == 0) {
+        ++checked;
+        EXPECT(barrier_kernel_splits(N / 256, N, K / 32, 32, 256, sc, sp) ==
+               barrier_kernel_splits(N / 256, N, K / 32, 32, 256, hc, hp));
+      }
+      if (failures > 20) return 1;
+    }
   if (failures) return 1;
   std::printf("skinny plan OK (%ld cases)\n", checked);
   return 0;

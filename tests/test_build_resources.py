@@ -35,7 +35,8 @@ def kernel_resources(src, outdir):
 @pytest.mark.skipif(HIPCC is None, reason="hipcc not installed")
 def test_hot_kernels_do_not_spill():
     files = [os.path.join(CSRC, f) for f in ("gemm_16b.hip", "gemm_i8.hip", "gemm_f32.hip",
-                                              "gemm_skinny.hip", "gemm_f32_small.hip", "probe.hip")]
+                                              "gemm_skinny.hip", "gemm_f32_small.hip", "probe.hip",
+                                              "probe_paired.hip")]
     with tempfile.TemporaryDirectory() as d, concurrent.futures.ThreadPoolExecutor(6) as pool:
         results = list(pool.map(lambda f: kernel_resources(f, d), files))
     spills = {k: v for r in results for k, v in r.items()}
@@ -43,5 +44,7 @@ def test_hot_kernels_do_not_spill():
     for name, n in spills.items():
         if re.search(r"EpiDequantX4ILb[01]ELb1", name):
             assert n <= 160, (name, n)     # accumulator-dump variants (a test aid)
+        elif "issue_cost_kernel" in name:
+            assert n <= 12, (name, n)      # (set-up values, spilled once outside the timed loop)
         else:
             assert n == 0, (name, n)

@@ -100,23 +100,3 @@ def test_kernel_family_selection(torch_gpu):
         c = h.gemm_i8_i32(a8, a8)
         assert (c.cpu().numpy() == 64).all()
     h.close()
-
-
-def test_matrix_core_probe(handle, torch_gpu):
-    """The measurement aid launches on the handle's stream, reports the operation count of one
-    launch, and rejects unknown kinds."""
-    import ctypes
-    ops = handle.probe_mfma("bf16", True, 10)
-    cus = torch_gpu.cuda.get_device_properties(0).multi_processor_count
-    assert ops == cus * 4 * 10 * 12 * 32768
-    assert handle.probe_mfma("i8", False, 10) == 2 * ops
-    assert handle.probe_mfma("bf16_16x16", False, 10) == ops // 2
-    assert handle.probe_mfma("i8_16x16", False, 10) == ops
-    torch_gpu.cuda.synchronize()
-    assert handle.last_kernel == "mfma_probe"
-    n = ctypes.c_int64(0)
-    assert handle.probe_mfma("f32", True, 10) == ops // 8
-    assert handle.lib.cigemm_probe_mfma(handle.raw, 7, 0, 10, ctypes.byref(n)) == Status.INVALID_VALUE
-    assert handle.lib.cigemm_probe_mfma(handle.raw, 0, 0, 0, ctypes.byref(n)) == Status.INVALID_VALUE
-    assert handle.lib.cigemm_probe_mfma(handle.raw, 0, 0, 10, None) == Status.SUCCESS
-    torch_gpu.cuda.synchronize()

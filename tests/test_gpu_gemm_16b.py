@@ -164,6 +164,9 @@ def test_config_8192(handle, torch_gpu, oracle, kind, parity_stats):
         "max_err_over_bound": float(allr.max()), "mean_err_over_bound": float(allr.mean()),
         "bound": "u_out*|ref64| + 2*K*2^-24*sum|a||b|, u_out = 2^-11 (fp16) / 2^-8 (bf16)"}
     assert (col_ratio <= 1.0).all()
+    # the maximum leaves a factor of six of room (observed 0.16 bf16 / 0.024 fp16); a systematic
+    # loss -- a k index dropped in some tile -- would move the mean (observed 0.018 / 0.0025)
+    assert allr.mean() <= 0.05, allr.mean()
     # Freivalds: C.x vs A.(B.x) in fp64 for +-1 vectors; output rounding errors are
     # independent with relative size u_out, so the projection error concentrates
     r = np.random.Generator(np.random.PCG64(5))
@@ -175,3 +178,40 @@ def test_config_8192(handle, torch_gpu, oracle, kind, parity_stats):
         scale = np.sqrt((Cf.astype(np.float64) ** 2).sum(axis=1))   # |row|_2
         assert (np.abs(lhs - rhs) <= 8 * u_out * scale).all()
     print(f"[{kind} 8192^3] worst sampled error = {worst:.3f} x bound")
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_config_8192_exact(handle, torch_gpu, oracle, kind, parity_stats):
+    """fp16 / bf16 8192^3 pinned exactly over the WHOLE matrix.  Inputs from {0, +-0.5, +-1, +-2}:
+    every product is a multiple of 1/4 of magnitude at most 4, every partial sum of up to 8192 of
+    them is below 2^17 quarter units, so fp32 accumulation is exact in ANY order and the one
+    correct output is narrow(exact sum).  The exact sums come from a float64 matrix product on
+    the host (exact for the same reason, in any blocking), tied to the oracle's own fp32 loop on
+    a stratified sample of rows and columns; the GPU result must equal their narrowing bit for
+    bit on all 8192 x 8192 entries.  One dropped, repeated or misplaced k index anywhere in the
+    four rounds of tiles changes entries by at least 1/4 and fails this."""
+    torch = torch_gpu
+    n = 8192
+    r = np.random.Generator(np.random.PCG64(21))
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    Af, Bf = r.choice(vals, size=(n, n)), r.choice(vals, size=(n, n))
+    narrow = oracle.f32_to_bf16 if kind == "bf16" else oracle.f32_to_f16
+    Ab, Bb = narrow(Af), narrow(Bf)
+    assert np.array_equal(widen(oracle, Ab, kind), Af)       # the inputs are exact in 16 bits
+    C = (handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16)(to_dev(torch, Ab, kind), to_dev(torch, Bb, kind))
+    assert "mfma" in handle.last_kernel and handle.last_plan == (256, 1)
+    Cb = bits(torch, C)
+    exact = Af.astype(np.float64) @ Bf.astype(np.float64)
+    assert np.abs(exact).max() < 65504 and np.array_equal(exact * 4, np.rint(exact * 4))
+    # the host product against the oracle's loop (k ascending, float accumulator), bit for bit
+    rows = np.array([0, 1, 31, 32, 255, 256, 257, 4095, 4096, 8190, 8191])
+    np.testing.assert_array_equal(oracle.gemm_f32(np.ascontiguousarray(Af[rows]), Bf),
+                                  exact[rows].astype(np.float32))
+    cols = np.array([0, 3, 4, 127, 128, 255, 256, 4097, 8191])
+    np.testing.assert_array_equal(oracle.gemm_f32(Af, np.ascontiguousarray(Bf[:, cols])),
+                                  exact[:, cols].astype(np.float32))
+    want = narrow(exact.astype(np.float32))
+    diff = int((Cb != want).sum())
+    parity_stats[f"C3_{kind}_8192_exact_inputs"] = {"kernel": handle.last_kernel, "entries": n * n,
+                                                    "entries_differing": diff}
+    assert diff == 0

@@ -1,28 +1,31 @@
-"""The instrumented launch of the tile kernel (cigemm_probe_tile_phases): it is the product
-kernel plus four timestamps per workgroup, so its output must equal the plain entry point's
-bit for bit, and the figures it reduces must be self-consistent."""
+"""The measurement aids of libcigemm_probe.so (include/cigemm_probe.h).  The instrumented launch
+of the tile kernel is the product kernel plus four timestamps per workgroup, so its output must
+equal the plain entry point's bit for bit, and the figures it reduces must be self-consistent;
+the register-resident loops report their operation counts and plausible cycle counts."""
 import numpy as np
 import pytest
 
 import cudaintro_amd as ci
+from cudaintro_amd import probe
 from gpu_util import to_dev
 
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("kind", ["bf16", "i8"])
+@pytest.mark.parametrize("kind", ["bf16", "f16", "i8"])
 @pytest.mark.parametrize("M,N,K", [(512, 512, 1024), (300, 272, 1008), (2048, 2048, 2048)])
 def test_probe_output_equals_plain_call_and_phases_add_up(handle, torch_gpu, oracle, rng, kind, M, N, K):
     torch = torch_gpu
-    if kind == "bf16":
+    if kind != "i8":
         # exact-arithmetic inputs: the plain call may split K or pick another tile height,
         # and only such inputs give the same bits in any summation order
         vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
-        a = to_dev(torch, oracle.f32_to_bf16(rng.choice(vals, size=(M, K))), "bf16")
-        b = to_dev(torch, oracle.f32_to_bf16(rng.choice(vals, size=(K, N))), "bf16")
-        out = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        narrow = oracle.f32_to_bf16 if kind == "bf16" else oracle.f32_to_f16
+        a = to_dev(torch, narrow(rng.choice(vals, size=(M, K))), kind)
+        b = to_dev(torch, narrow(rng.choice(vals, size=(K, N))), kind)
+        out = torch.zeros((M, N), dtype=a.dtype, device="cuda")
         with handle.algo(ci.ALGO_TILE):
-            want = handle.gemm_bf16(a, b)
+            want = (handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16)(a, b)
     else:
         a = torch.from_numpy(rng.integers(-127, 128, size=(M, K), dtype=np.int8)).cuda()
         b = torch.from_numpy(rng.integers(-127, 128, size=(K, N), dtype=np.int8)).cuda()
@@ -30,8 +33,10 @@ def test_probe_output_equals_plain_call_and_phases_add_up(handle, torch_gpu, ora
         with handle.algo(ci.ALGO_TILE):
             want = handle.gemm_i8_i32(a, b, ci.B_KN)
     for paired, rows, min_cycles in ((False, 256, 1024), (True, 128, 512)):
+        if paired and kind == "f16":
+            continue
         out.zero_()
-        ph = handle.probe_tile_phases(a, b, out, paired=paired)
+        ph = probe.tile_phases(handle, a, b, out, paired=paired)
         assert handle.last_kernel == "tile_phase_probe"
         assert torch.equal(out.view(torch.uint8), want.view(torch.uint8))
         tiles = -(-M // rows) * -(-N // 256)
@@ -50,4 +55,48 @@ def test_probe_rejects_bad_arguments(handle, torch_gpu):
     b = torch.zeros((60, 64), dtype=torch.bfloat16, device="cuda")
     out = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ci.CigemmError, match="NOT_SUPPORTED"):
-        handle.probe_tile_phases(a, b, out)
+        probe.tile_phases(handle, a, b, out)
+
+
+def test_matrix_core_probe(handle, torch_gpu):
+    """The register-resident loop launches on the handle's stream, reports the operation count of
+    one launch, and rejects unknown kinds."""
+    import ctypes
+    from cudaintro_amd import Status
+    lib = probe.load_library()
+    ops = probe.mfma(handle, "bf16", True, 10)
+    cus = torch_gpu.cuda.get_device_properties(0).multi_processor_count
+    assert ops == cus * 4 * 10 * 12 * 32768
+    assert probe.mfma(handle, "i8", False, 10) == 2 * ops
+    assert probe.mfma(handle, "bf16_16x16", False, 10) == ops // 2
+    assert probe.mfma(handle, "i8_16x16", False, 10) == ops
+    torch_gpu.cuda.synchronize()
+    assert handle.last_kernel == "mfma_probe"
+    n = ctypes.c_int64(0)
+    assert probe.mfma(handle, "f32", True, 10) == ops // 8
+    assert lib.cigemm_probe_mfma(handle.raw, 7, 0, 10, ctypes.byref(n)) == Status.INVALID_VALUE
+    assert lib.cigemm_probe_mfma(handle.raw, 0, 0, 0, ctypes.byref(n)) == Status.INVALID_VALUE
+    assert lib.cigemm_probe_mfma(handle.raw, 0, 0, 10, None) == Status.SUCCESS
+    torch_gpu.cuda.synchronize()
+
+
+def test_issue_cost_probe(handle, torch_gpu):
+    """32 matrix instructions of 8 passes of 4 cycles cannot issue in fewer than 1024 cycles; the
+    companions (LDS-DMA, fragment reads, a barrier) can only add to that; bad arguments are
+    refused before anything is launched."""
+    import ctypes
+    from cudaintro_amd import Status
+    lib = probe.load_library()
+    cus = torch_gpu.cuda.get_device_properties(0).multi_processor_count
+    base = probe.issue_cost(handle, 0, 0, False, 4, 2000)
+    assert handle.last_kernel == "issue_cost_probe"
+    assert 1024 <= base["cycles_per_stage"] < 1100, base
+    assert base["cycles_per_stage"] <= base["cycles_per_stage_slowest_wave"]
+    assert 0.05 < base["clock_ghz"] < 3.0 and base["launch_us"] > 0
+    full = probe.issue_cost(handle, 8, 24, True, cus, 2000)
+    assert base["cycles_per_stage"] <= full["cycles_per_stage"] < 4 * 1024, full
+    res = (ctypes.c_double * 4)()
+    for bad in ((3, 0, 0, 4, 10), (0, 12, 0, 4, 10), (0, 0, 2, 4, 10), (0, 0, 0, 0, 10),
+                (0, 0, 0, cus + 1, 10), (0, 0, 0, 4, 0)):
+        assert lib.cigemm_probe_issue_cost(handle.raw, *bad, res) == Status.INVALID_VALUE
+    assert lib.cigemm_probe_issue_cost(handle.raw, 0, 0, 0, 4, 10, None) == Status.INVALID_VALUE

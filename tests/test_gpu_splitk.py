@@ -116,3 +116,45 @@ def test_splitk_workspace_reuse_with_alternating_inputs(handle, torch_gpu, oracl
             got = handle.gemm_i8_i32(a, b, ci.B_KN).cpu().numpy()
         assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
         np.testing.assert_array_equal(got, want, err_msg=f"call {i}")
+
+
+def test_handle_recovers_after_a_failed_launch(torch_gpu, oracle, rng):
+    """A split-K kernel that did not run to its end leaves arrival counters or exchange words
+    non-zero.  The state is forged from the host here (a copy into the workspace; every kernel
+    runs normally): a handle marked as a failed launch marks it clears them by itself before
+    its next GEMM, and cigemmResetWorkspace does it on request."""
+    from cudaintro_amd import probe
+    torch = torch_gpu
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    cases = []
+    # four K ranges per slab (partials and arrival counters); two ranges (one exchange word per
+    # pair of outputs)
+    for (M, N, K) in ((8, 8192, 8192), (4, 13824, 5120)):
+        x = to_dev(torch, oracle.f32_to_bf16(rng.choice(vals, size=(M, K))), "bf16")
+        w = to_dev(torch, oracle.f32_to_bf16(rng.choice(vals, size=(K, N)) * (rng.random((K, N)) < 0.1)), "bf16")
+        cases.append((x, w))
+    with ci.Handle() as h:
+        want = []
+        for x, w in cases:
+            want.append(h.gemm_bf16(x, w).clone())
+            assert "skinny" in h.last_kernel, h.last_kernel
+        torch.cuda.synchronize()
+
+        def run_all():
+            outs = []
+            for x, w in cases:
+                y = torch.full((x.shape[0], w.shape[1]), 3.0, dtype=torch.bfloat16, device="cuda")
+                outs.append(h.gemm_bf16(x, w, out=y))
+            torch.cuda.synchronize()
+            return outs
+
+        # the forged state matters: without a reset the same calls come out wrong (no kernel
+        # waits on these words, so nothing can hang: an output is left unwritten or mis-summed)
+        probe.dirty_workspace(h, 8192, 7, mark_dirty=False)
+        assert not all(torch.equal(a, b) for a, b in zip(run_all(), want))
+        h.reset_workspace()
+        assert all(torch.equal(a, b) for a, b in zip(run_all(), want))
+        # what a call ending in CIGEMM_STATUS_EXECUTION_FAILED records: cleared without being asked
+        probe.dirty_workspace(h, 8192, 7, mark_dirty=True)
+        assert all(torch.equal(a, b) for a, b in zip(run_all(), want))
+        assert all(torch.equal(a, b) for a, b in zip(run_all(), want))
