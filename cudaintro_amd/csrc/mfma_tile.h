@@ -672,8 +672,16 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   constexpr int NMFMA = 4 * MT * Math::SUBSTEPS;       // MFMAs per k-step
   constexpr int READS_PER_SLOT = (NREAD + NMFMA - 1) / NMFMA;
   static_assert(DMA_A % 2 == 0, "an A pair is issued in two halves");
-  constexpr int DMA_PER_SLOT =
-      ((BPAIR ? (DMA_A > DMA_B ? DMA_A : DMA_B) : DMA_B + DMA_A / 2) + NMFMA - 1) / NMFMA;
+  // DMA instruction d of the NDMA a k-step issues goes into MFMA slot d * NMFMA / NDMA: spread
+  // evenly over the k-step.  The four waves leave the barrier together, and a compute unit's one
+  // address path takes about 16 cycles per 1 KiB instruction: issued back to back, one per
+  // 32-cycle matrix instruction from every wave, they queue up and stall the waves' issue (a
+  // register-resident loop with the stage's 8 instructions in its first 8 slots after a barrier
+  // takes 1130 cycles per stage, in every second slot 1033, without any 1029).
+  // (first and one-past-last DMA instruction of slot sl)
+  constexpr auto dma_begin_of_slot = [](int sl, int ndma) constexpr {
+    return ndma <= NMFMA ? (sl * ndma + NMFMA - 1) / NMFMA : sl * ((ndma + NMFMA - 1) / NMFMA);
+  };
   struct Frags {
     u32x4 a[BPAIR ? MT + 4 : MT];
     typename BT::piece_t b[BPAIR ? 1 : BT::NREADS];
@@ -750,15 +758,34 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   // even stages issue the A pair of stages s+4, s+5 (same slot rule), odd stages the B pair
   // of stages s+3, s+4 (its slot, one of two, is the one this stage stops reading): the
   // instructions of a stage pair are spread over both of its stages.
-  auto stage = [&](int s, auto par_const, auto steady_const) {
+  // PHASE = s mod 12 when the caller knows it (the rings have periods of 4 and 6 stages), else
+  // -1.  With a known phase every ring slot of the stage is a constant: the LDS addresses of its
+  // fragment reads become a loop-invariant lane offset plus an immediate, the DMA destinations
+  // immediates too, and the stage carries no ring arithmetic at all.  With one wave per SIMD
+  // every instruction costs that wave four issue cycles, and only about seven fit under one
+  // matrix instruction: the 12-stage body takes 1060 cycles per stage where the one that
+  // computes its slots takes 1200.
+  auto stage = [&](int s, auto par_const, auto steady_const, auto phase_const) {
     constexpr int PAR = decltype(par_const)::value;
+    constexpr int PHASE = decltype(phase_const)::value;
+    static_assert(PHASE < 0 || (PHASE & 1) == PAR, "the phase fixes the parity");
     constexpr int NDMA = BPAIR ? (PAR ? DMA_B : DMA_A) : DMA_B + DMA_A / 2;
+    int slot_c = slot, next_slot_c = next_slot, dma_slot_c = dma_slot;
+    int pslot_c = pslot, next_pslot_c = next_pslot, dma_pslot_c = dma_pslot;
+    if constexpr (PHASE >= 0) {
+      slot_c = BPAIR ? (PHASE / 2) % 2 : PHASE % NSTAGES;
+      next_slot_c = BPAIR ? 1 - slot_c : (PHASE + 1) % NSTAGES;
+      dma_slot_c = (PHASE + DIST) % NSTAGES;
+      pslot_c = (PHASE / 2) % 3;
+      next_pslot_c = (PHASE / 2 + 1) % 3;
+      dma_pslot_c = (PHASE / 2 + 2) % 3;
+    }
 #pragma unroll
     for (int sl = 0; sl < NMFMA; ++sl) {
       mfma_piece(f0, sl);
 #pragma unroll
       for (int r = sl * READS_PER_SLOT; r < (sl + 1) * READS_PER_SLOT; ++r)
-        if (r < NREAD) read_piece(f1, slot, pslot, PAR, 1, r);
+        if (r < NREAD) read_piece(f1, slot_c, pslot_c, PAR, 1, r);
       __builtin_amdgcn_sched_barrier(0);
     }
     if (BPAIR) {
@@ -784,57 +811,79 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
 #pragma unroll
       for (int r = sl * READS_PER_SLOT; r < (sl + 1) * READS_PER_SLOT; ++r)
         if (r < NREAD)
-          read_piece(f0, BPAIR ? (PAR ? next_slot : slot) : next_slot, PAR ? next_pslot : pslot,
+          read_piece(f0, BPAIR ? (PAR ? next_slot_c : slot_c) : next_slot_c, PAR ? next_pslot_c : pslot_c,
                      PAR ^ 1, 0, r);
 #pragma unroll
-      for (int d = sl * DMA_PER_SLOT; d < (sl + 1) * DMA_PER_SLOT; ++d)
-        if (d < NDMA) {
+      for (int dd = 0; dd < (NDMA + NMFMA - 1) / NMFMA; ++dd) {  // (a constant trip count)
+        const int d = dma_begin_of_slot(sl, NDMA) + dd;
+        if (d < dma_begin_of_slot(sl + 1, NDMA) && d < NDMA) {
           if (BPAIR) {
             if (PAR)
-              dma_piece(s + DIST, slot, dma_pslot, d, steady_const);               // B pair
+              dma_piece(s + DIST, slot_c, dma_pslot_c, d, steady_const);           // B pair
             else
-              dma_piece(s + DIST + 1, slot, dma_pslot, DMA_B + d, steady_const);   // A pair
+              dma_piece(s + DIST + 1, slot_c, dma_pslot_c, DMA_B + d, steady_const);  // A pair
           } else if (d < DMA_B) {
-            dma_piece(s + DIST, dma_slot, dma_pslot, d, steady_const);             // B[s+3]
+            dma_piece(s + DIST, dma_slot_c, dma_pslot_c, d, steady_const);         // B[s+3]
           } else {
             // half of the A pair the DMA is filling: stages s+4, s+5 seen from an even stage,
             // s+3, s+4 from the odd stage after it
-            dma_piece(PAR ? s + DIST : s + DIST + 1, dma_slot, dma_pslot,
+            dma_piece(PAR ? s + DIST : s + DIST + 1, dma_slot_c, dma_pslot_c,
                       d + (PAR ? DMA_A / 2 : 0), steady_const);
           }
         }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (BPAIR) {
-      if (PAR) {
-        const int tmp = slot;
+    if constexpr (PHASE < 0) {
+      if (BPAIR) {
+        if (PAR) {
+          const int tmp = slot;
+          slot = next_slot;
+          next_slot = tmp;
+        }
+      } else {
         slot = next_slot;
-        next_slot = tmp;
+        next_slot = next_slot + 1 == NSTAGES ? 0 : next_slot + 1;
+        dma_slot = dma_slot + 1 == NSTAGES ? 0 : dma_slot + 1;
       }
-    } else {
-      slot = next_slot;
-      next_slot = next_slot + 1 == NSTAGES ? 0 : next_slot + 1;
-      dma_slot = dma_slot + 1 == NSTAGES ? 0 : dma_slot + 1;
-    }
-    if (PAR) {
-      pslot = next_pslot;
-      next_pslot = next_pslot + 1 == 3 ? 0 : next_pslot + 1;
-      dma_pslot = dma_pslot + 1 == 3 ? 0 : dma_pslot + 1;
+      if (PAR) {
+        pslot = next_pslot;
+        next_pslot = next_pslot + 1 == 3 ? 0 : next_pslot + 1;
+        dma_pslot = dma_pslot + 1 == 3 ? 0 : dma_pslot + 1;
+      }
     }
   };
   // Steady part: every stage the DMA reaches (up to s + 5) exists and its pair is whole.
   const int steady_end = (pair_valid < 8 && !(KTS & 1)) ? KTS - 2 : KTS;
+  typedef std::integral_constant<int, -1> any_phase_t;
   int s = 0;
+  // twelve stages at a time with every ring slot a constant (the slot variables keep their
+  // values of phase 0 meanwhile: s stays a multiple of 12) ...
+  for (; s + 11 + 5 < steady_end; s += 12) {
+    stage(s, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 0>{});
+    stage(s + 1, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 1>{});
+    stage(s + 2, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 2>{});
+    stage(s + 3, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 3>{});
+    stage(s + 4, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 4>{});
+    stage(s + 5, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 5>{});
+    stage(s + 6, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 6>{});
+    stage(s + 7, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 7>{});
+    stage(s + 8, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 8>{});
+    stage(s + 9, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 9>{});
+    stage(s + 10, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 10>{});
+    stage(s + 11, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 11>{});
+  }
+  // ... then the rest of the steady part and the drain, with the slots advanced at run time
   for (; s + 5 < steady_end; s += 2) {
-    stage(s, std::integral_constant<int, 0>{}, steady_t{});
-    stage(s + 1, std::integral_constant<int, 1>{}, steady_t{});
+    stage(s, std::integral_constant<int, 0>{}, steady_t{}, any_phase_t{});
+    stage(s + 1, std::integral_constant<int, 1>{}, steady_t{}, any_phase_t{});
   }
   for (; s + 1 < KTS; s += 2) {
-    stage(s, std::integral_constant<int, 0>{}, drain_t{});
-    stage(s + 1, std::integral_constant<int, 1>{}, drain_t{});
+    stage(s, std::integral_constant<int, 0>{}, drain_t{}, any_phase_t{});
+    stage(s + 1, std::integral_constant<int, 1>{}, drain_t{}, any_phase_t{});
   }
   // odd stage count: the last one
-  if (KTS & 1) stage(KTS - 1, std::integral_constant<int, 0>{}, drain_t{});
+  if (KTS & 1) stage(KTS - 1, std::integral_constant<int, 0>{}, drain_t{}, any_phase_t{});
   wait_vmcnt(std::integral_constant<int, 0>{});  // no DMA outlives the main loop
   __syncthreads();  // ... for any wave, and every wave is done reading the ring
   stamp(2);

@@ -3,6 +3,7 @@
 // actually holds under this load.  Sustained rate depends on the operand data (the chip is
 // power limited), so the probe runs on constant or on pseudo-random operand bits.
 #include <algorithm>
+#include <type_traits>
 #include <vector>
 
 #include "cigemm_probe.h"
@@ -112,10 +113,27 @@ __global__ __launch_bounds__(256, 1) void mfma_probe_kernel(float* __restrict__ 
 // one DMA) is closed by a scheduling fence.
 typedef __attribute__((address_space(3))) i16x4 probe_lds_i16x4;
 
-template <int NDMA, int NLDS, int BARRIER>
+// Where the DMA instructions go: instruction d of wave w sits in slot (w * WOFF + d * STRIDE)
+// mod 32 of the 32 slots between one barrier and the next (slots 0..15: the k-step after the
+// barrier, 16..31: the k-step before the next one).  STRIDE 1, WOFF 0 is the product kernel's
+// placement before it was spread: every wave issues its instructions back to back right after
+// the barrier, so that the compute unit's one address path sees all of them at once.
+constexpr bool dma_in_slot(int g, int off, int stride, int ndma) {
+  for (int d = 0; d < ndma; ++d)
+    if ((off + d * stride) % 32 == g) return true;
+  return false;
+}
+constexpr int dma_index(int g, int off, int stride, int ndma) {
+  for (int d = 0; d < ndma; ++d)
+    if ((off + d * stride) % 32 == g) return d;
+  return 0;
+}
+
+template <int NDMA, int NLDS, int BARRIER, int STRIDE, int WOFF, int MFMA>
 __global__ __launch_bounds__(256, 1) void issue_cost_kernel(const char* __restrict__ src,
                                                             uint64_t* __restrict__ stamps,
-                                                            float* __restrict__ sink, int iters) {
+                                                            float* __restrict__ sink, int iters,
+                                                            int src_span) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int t = threadIdx.x, l = t & 63;
   const int w = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -131,7 +149,11 @@ __global__ __launch_bounds__(256, 1) void issue_cost_kernel(const char* __restri
     *reinterpret_cast<u32x4*>(rd + i) = v;
   }
   __syncthreads();
-  const char* my_src = src + ((size_t)blockIdx.x * 4 + w) * 8192;
+  // the wave's DMA source: `src_span` bytes walked 8 KiB per stage, round and round (8 KiB: the
+  // same lines every stage, served by the vector L1; more than the L1 holds: by the L2)
+  const char* const my_src0 = src + ((size_t)blockIdx.x * 4 + w) * (size_t)src_span;
+  const char* my_src = my_src0;
+  int src_off = 0;
   const uint32_t voff = (uint32_t)l * 16;
   struct Frags {
     u32x4 a[4];
@@ -157,7 +179,17 @@ __global__ __launch_bounds__(256, 1) void issue_cost_kernel(const char* __restri
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  uint32_t fold = 0;  // without matrix instructions: what consumes the fragments instead
   auto mfma_piece = [&](const Frags& f, int m) {
+    if (!MFMA) {
+      if (m == 15 && NLDS) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) fold ^= f.a[r][0];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) fold ^= f.b[r][0];
+      }
+      return;
+    }
     const int j = m / 4;
     const int i = (j & 1) ? 3 - m % 4 : m % 4;
     const u32x4 bfrag = __builtin_shufflevector(f.b[2 * j], f.b[2 * j + 1], 0, 1, 2, 3);
@@ -165,36 +197,52 @@ __global__ __launch_bounds__(256, 1) void issue_cost_kernel(const char* __restri
                                                         __builtin_bit_cast(bf16x8, f.a[i]),
                                                         acc[i][j], 0, 0, 0);
   };
+  auto dma = [&](int d) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(dma_dst + d * 1024), "v"(voff), "s"(my_src)
+                 : "m0");
+  };
   uint64_t t0 = 0, r0 = 0;
   if (l == 0) {
     t0 = __builtin_amdgcn_s_memtime();
     r0 = __builtin_amdgcn_s_memrealtime();
   }
-  for (int it = 0; it < iters; ++it) {
+  auto run = [&](auto off_const) {
+    constexpr int OFF = decltype(off_const)::value;
+    for (int it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int sl = 0; sl < 16; ++sl) {
-      mfma_piece(f0, sl);
-      if (NLDS && sl < 12) read_piece(f1, 1, sl);
+      for (int sl = 0; sl < 16; ++sl) {
+        mfma_piece(f0, sl);
+        if (NLDS && sl < 12) read_piece(f1, 1, sl);
+        if (dma_in_slot(16 + sl, OFF, STRIDE, NDMA)) dma(dma_index(16 + sl, OFF, STRIDE, NDMA));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // (as in the product: everything but the DMA of the last two stages has landed)
+      if (NDMA) __builtin_amdgcn_s_waitcnt(0x0f70 | ((2 * NDMA) & 15) | (((2 * NDMA) >> 4) << 14));
+      if (BARRIER) __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
-    }
-    // (as in the product: everything but the DMA of the last two stages has landed)
-    if (NDMA) __builtin_amdgcn_s_waitcnt(0x0f70 | ((2 * NDMA) & 15) | (((2 * NDMA) >> 4) << 14));
-    if (BARRIER) __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int sl = 0; sl < 16; ++sl) {
-      mfma_piece(f1, sl);
-      if (NLDS && sl < 12) read_piece(f0, 0, sl);
-      if (sl < NDMA)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     :
-                     : "s"(dma_dst + sl * 1024), "v"(voff), "s"(my_src)
-                     : "m0");
-      __builtin_amdgcn_sched_barrier(0);
+      for (int sl = 0; sl < 16; ++sl) {
+        mfma_piece(f1, sl);
+        if (NLDS && sl < 12) read_piece(f0, 0, sl);
+        if (dma_in_slot(sl, OFF, STRIDE, NDMA)) dma(dma_index(sl, OFF, STRIDE, NDMA));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      asm volatile("" ::: "memory");
+      src_off = src_off + 8192 < src_span ? src_off + 8192 : 0;
+      my_src = my_src0 + src_off;
     }
-    asm volatile("" ::: "memory");
-  }
+  };
+  if (WOFF == 0 || w == 0)
+    run(std::integral_constant<int, 0>{});
+  else if (w == 1)
+    run(std::integral_constant<int, WOFF>{});
+  else if (w == 2)
+    run(std::integral_constant<int, 2 * WOFF>{});
+  else
+    run(std::integral_constant<int, 3 * WOFF>{});
   if (l == 0) {
     uint64_t* p = stamps + ((size_t)blockIdx.x * 4 + w) * 4;
     p[0] = t0;
@@ -210,7 +258,7 @@ __global__ __launch_bounds__(256, 1) void issue_cost_kernel(const char* __restri
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) sum += acc[i][j][e];
-  sink[blockIdx.x * 256 + t] = sum;
+  sink[blockIdx.x * 256 + t] = sum + (float)(fold & 1);
 }
 
 // Microseconds per tick of the constant-rate counter s_memrealtime reads.
@@ -225,14 +273,14 @@ double wall_tick_us(int device) {
 
 constexpr int ISSUE_LDS_BYTES = 4 * 16384;
 
-template <int NDMA, int NLDS, int BARRIER>
+template <int NDMA, int NLDS, int BARRIER, int STRIDE = 1, int WOFF = 0, int MFMA = 1>
 void launch_issue_cost(cigemmContext* ctx, int grid, const char* src, uint64_t* stamps, float* sink,
-                       int iters) {
-  auto kern = issue_cost_kernel<NDMA, NLDS, BARRIER>;
+                       int iters, int src_span) {
+  auto kern = issue_cost_kernel<NDMA, NLDS, BARRIER, STRIDE, WOFF, MFMA>;
   static std::atomic<uint64_t> lds_set{0};
   if (!ensure_dynamic_lds(ctx, (const void*)kern, ISSUE_LDS_BYTES, lds_set)) return;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), ISSUE_LDS_BYTES, ctx->stream, src, stamps, sink,
-                     iters);
+                     iters, src_span);
 }
 
 }  // namespace
@@ -271,35 +319,84 @@ extern "C" cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t h, int kind, int rand
 }
 
 extern "C" cigemmStatus_t cigemm_probe_issue_cost(cigemmHandle_t h, int n_dma, int n_lds_reads,
-                                                  int barrier, int workgroups, int iters,
+                                                  int barrier, int placement, int mfma,
+                                                  int src_kib_per_wave, int workgroups, int iters,
                                                   double* result) {
   const char* name = "cigemm_probe_issue_cost";
   if (!h || h->magic != kCtxMagic) return CIGEMM_STATUS_NOT_INITIALIZED;
   const int cus = h->num_cus > 0 ? h->num_cus : 256;
   if ((n_dma != 0 && n_dma != 2 && n_dma != 4 && n_dma != 8) ||
-      (n_lds_reads != 0 && n_lds_reads != 24) || (barrier != 0 && barrier != 1) || workgroups < 1 ||
+      (n_lds_reads != 0 && n_lds_reads != 24) || (barrier != 0 && barrier != 1) || placement < 0 ||
+      placement > 7 || (placement > 0 && (n_dma != 8 || (mfma && n_lds_reads != 24))) ||
+      (mfma != 0 && mfma != 1) ||
+      (!mfma && (placement > 1 || (n_dma != 0 && n_dma != 8))) || src_kib_per_wave < 8 ||
+      src_kib_per_wave % 8 || src_kib_per_wave > 1024 || workgroups < 1 ||
       workgroups > cus || iters <= 0 || iters > (1 << 22) || !result)
     return fail(h, CIGEMM_STATUS_INVALID_VALUE,
-                "%s: n_dma %d (0, 2, 4, 8), n_lds_reads %d (0, 24), barrier %d, workgroups %d "
-                "(1..%d), iters %d", name, n_dma, n_lds_reads, barrier, workgroups, cus, iters);
-  // workspace: stamps (32 bytes per wave), the sink, then 8 KiB of DMA source per wave
+                "%s: n_dma %d (0, 2, 4, 8), n_lds_reads %d (0, 24), barrier %d, placement %d (0..7; "
+                "above 0 only with n_dma 8 and n_lds_reads 24), mfma %d (0 only with placement 0 or 1 "
+                "and n_dma 0 or 8), src_kib_per_wave %d (8..1024, multiple of 8), workgroups %d "
+                "(1..%d), iters %d",
+                name, n_dma, n_lds_reads, barrier, placement, mfma, src_kib_per_wave, workgroups, cus,
+                iters);
+  // workspace: stamps (32 bytes per wave), the sink, then the DMA source of every wave
+  const int src_span = src_kib_per_wave * 1024;
   const size_t stamp_bytes = (size_t)workgroups * 4 * 32, sink_bytes = (size_t)workgroups * 1024;
   const size_t src_off = (stamp_bytes + sink_bytes + 4095) & ~(size_t)4095;
-  if (!h->workspace || src_off + (size_t)workgroups * 4 * 8192 > h->ws_partial_bytes)
-    return fail(h, CIGEMM_STATUS_ALLOC_FAILED, "%s: workspace too small", name);
+  if (!h->workspace || src_off + (size_t)workgroups * 4 * (size_t)src_span > h->ws_partial_bytes)
+    return fail(h, CIGEMM_STATUS_NOT_SUPPORTED,
+                "%s: %d workgroups x 4 waves x %d KiB of DMA source exceed the workspace", name,
+                workgroups, src_kib_per_wave);
   char* ws = static_cast<char*>(h->workspace);
   uint64_t* stamps = reinterpret_cast<uint64_t*>(ws);
   float* sink = reinterpret_cast<float*>(ws + stamp_bytes);
   const char* src = ws + src_off;
-#define CIG_IC(D, L, B) launch_issue_cost<D, L, B>(h, workgroups, src, stamps, sink, iters)
+#define CIG_IC(D, L, B) launch_issue_cost<D, L, B>(h, workgroups, src, stamps, sink, iters, src_span)
 #define CIG_IC_B(D, L) do { if (barrier) CIG_IC(D, L, 1); else CIG_IC(D, L, 0); } while (0)
 #define CIG_IC_L(D) do { if (n_lds_reads) CIG_IC_B(D, 24); else CIG_IC_B(D, 0); } while (0)
-  switch (n_dma) {
-    case 0: CIG_IC_L(0); break;
-    case 2: CIG_IC_L(2); break;
-    case 4: CIG_IC_L(4); break;
-    default: CIG_IC_L(8); break;
+#define CIG_IC_P(S, W)                                                                   \
+  do {                                                                                   \
+    if (barrier)                                                                         \
+      launch_issue_cost<8, 24, 1, S, W>(h, workgroups, src, stamps, sink, iters, src_span); \
+    else                                                                                 \
+      launch_issue_cost<8, 24, 0, S, W>(h, workgroups, src, stamps, sink, iters, src_span); \
+  } while (0)
+#define CIG_IC_N(D, L, S)                                                                        \
+  do {                                                                                           \
+    if (barrier)                                                                                 \
+      launch_issue_cost<D, L, 1, S, 0, 0>(h, workgroups, src, stamps, sink, iters, src_span);    \
+    else                                                                                         \
+      launch_issue_cost<D, L, 0, S, 0, 0>(h, workgroups, src, stamps, sink, iters, src_span);    \
+  } while (0)
+  if (!mfma) {  // the stage's memory instructions alone, 32-cycle slots left empty
+    if (n_dma == 8 && n_lds_reads) {
+      if (placement) CIG_IC_N(8, 24, 2); else CIG_IC_N(8, 24, 1);
+    } else if (n_dma == 8) {
+      if (placement) CIG_IC_N(8, 0, 2); else CIG_IC_N(8, 0, 1);
+    } else if (n_lds_reads) {
+      CIG_IC_N(0, 24, 1);
+    } else {
+      CIG_IC_N(0, 0, 1);
+    }
+  } else
+  switch (placement) {
+    case 1: CIG_IC_P(2, 0); break;   // every second slot of the k-step after the barrier
+    case 2: CIG_IC_P(2, 1); break;   // ... waves 1 and 3 on the odd slots
+    case 3: CIG_IC_P(4, 0); break;   // every fourth slot, over both k-steps
+    case 4: CIG_IC_P(4, 1); break;   // ... wave w one slot after wave w - 1
+    case 5: CIG_IC_P(1, 4); break;   // back to back, wave w four slots after wave w - 1
+    case 6: CIG_IC_P(1, 8); break;   // back to back, wave w eight slots after wave w - 1
+    case 7: CIG_IC_P(2, 8); break;   // every second slot, wave w eight slots after wave w - 1
+    default:
+      switch (n_dma) {
+        case 0: CIG_IC_L(0); break;
+        case 2: CIG_IC_L(2); break;
+        case 4: CIG_IC_L(4); break;
+        default: CIG_IC_L(8); break;
+      }
   }
+#undef CIG_IC_P
+#undef CIG_IC_N
 #undef CIG_IC_L
 #undef CIG_IC_B
 #undef CIG_IC

@@ -20,7 +20,7 @@ _gemm = [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]
 # name -> (restype, argtypes); must list every symbol include/cigemm_probe.h declares.
 SIGNATURES = {
     "cigemm_probe_mfma": (_ci, [_vp, _ci, _ci, _ci, C.POINTER(C.c_int64)]),
-    "cigemm_probe_issue_cost": (_ci, [_vp, _ci, _ci, _ci, _ci, _ci, C.POINTER(C.c_double)]),
+    "cigemm_probe_issue_cost": (_ci, [_vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci, _ci, C.POINTER(C.c_double)]),
     "cigemm_probe_tile_phases": (_ci, [_vp, _ci, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64,
                                        C.POINTER(C.c_double)]),
     "cigemm_probe_gemm_bf16_paired": (_ci, _gemm),
@@ -68,11 +68,12 @@ def mfma(h: Handle, kind: str, random_bits: bool, iters: int) -> int:
     return ops.value
 
 
-def issue_cost(h: Handle, n_dma: int, n_lds_reads: int, barrier: bool, workgroups: int, iters: int):
+def issue_cost(h: Handle, n_dma: int, n_lds_reads: int, barrier: bool, workgroups: int, iters: int,
+               placement: int = 0, mfma: bool = True, src_kib_per_wave: int = 8):
     """Cycles per 32-matrix-instruction stage with the given companions; see cigemm_probe.h."""
     res = (C.c_double * 4)()
-    _check(h, load_library().cigemm_probe_issue_cost(h.raw, n_dma, n_lds_reads, int(barrier), workgroups,
-                                                     iters, res), "cigemm_probe_issue_cost")
+    _check(h, load_library().cigemm_probe_issue_cost(h.raw, n_dma, n_lds_reads, int(barrier), placement,
+                                                     int(mfma), src_kib_per_wave, workgroups, iters, res), "cigemm_probe_issue_cost")
     return dict(zip(("cycles_per_stage", "cycles_per_stage_slowest_wave", "clock_ghz", "launch_us"), list(res)))
 
 

@@ -38,12 +38,27 @@ CIGEMM_API cigemmStatus_t cigemm_probe_mfma(cigemmHandle_t handle, int kind, int
  *   n_lds_reads  LDS fragment reads (0 or 24: 8 of 16 bytes and 16 transposing 8-byte ones,
  *                the product's count per stage), whose results feed the next stage's matrix
  *                instructions,
- *   barrier      0 / 1 workgroup barriers per stage (the product has one).
+ *   barrier      0 / 1 workgroup barriers per stage (the product has one),
+ *   placement    where the DMA instructions sit among the 32 slots between one barrier and the
+ *                next (a slot = one matrix instruction; 0..15 the k-step after the barrier):
+ *                0 = the first n_dma slots after the barrier, every wave alike; 1 = every second
+ *                slot; 2 = every second slot, waves 1 and 3 on the odd ones; 3 = every fourth
+ *                slot over both k-steps; 4 = the same, wave w one slot after wave w - 1; 5, 6 =
+ *                back to back, wave w four / eight slots after wave w - 1; 7 = every second
+ *                slot, wave w eight slots after wave w - 1 (1..7 need n_dma 8, n_lds_reads 24),
+ *   mfma         1 = as described; 0 = the same loop without its matrix instructions (their
+ *                slots stay empty; the fragments are consumed by one vector instruction each):
+ *                what the stage's memory instructions take by themselves (placement 0 or 1,
+ *                n_dma 0 or 8),
+ *   src_kib_per_wave  bytes of DMA source a wave walks through, 8 KiB per stage, round and
+ *                round: 8 = the same lines every stage (vector-L1 hits), 32 and more = lines
+ *                the L1 no longer holds (served by the L2, as the product's are).
  * Synchronises the stream.  result[0..3] receive: shader cycles per stage, averaged over the
  * waves; the slowest wave's; the shader clock (GHz) held meanwhile; microseconds per launch
  * from the first wave's start to the last wave's end. */
 CIGEMM_API cigemmStatus_t cigemm_probe_issue_cost(cigemmHandle_t handle, int n_dma,
-                                                  int n_lds_reads, int barrier, int workgroups,
+                                                  int n_lds_reads, int barrier, int placement,
+                                                  int mfma, int src_kib_per_wave, int workgroups,
                                                   int iters, double* result);
 
 /* Runs ONE launch of the 256-row, four-wave LDS-tiled matrix-core kernel (the product kernel

@@ -66,7 +66,7 @@ def test_probe_library_is_separate_and_matches_its_header():
     assert sorted(probe.SIGNATURES) == names
     # null handle: a status code, never a crash
     assert lib.cigemm_probe_mfma(None, 0, 0, 1, None) == cigemm.Status.NOT_INITIALIZED
-    assert lib.cigemm_probe_issue_cost(None, 0, 0, 0, 1, 1, None) == cigemm.Status.NOT_INITIALIZED
+    assert lib.cigemm_probe_issue_cost(None, 0, 0, 0, 0, 1, 8, 1, 1, None) == cigemm.Status.NOT_INITIALIZED
     assert lib.cigemm_probe_dirty_workspace(None, 0, 0, 0) == cigemm.Status.NOT_INITIALIZED
 
 

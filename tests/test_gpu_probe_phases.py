@@ -96,7 +96,19 @@ def test_issue_cost_probe(handle, torch_gpu):
     full = probe.issue_cost(handle, 8, 24, True, cus, 2000)
     assert base["cycles_per_stage"] <= full["cycles_per_stage"] < 4 * 1024, full
     res = (ctypes.c_double * 4)()
-    for bad in ((3, 0, 0, 4, 10), (0, 12, 0, 4, 10), (0, 0, 2, 4, 10), (0, 0, 0, 0, 10),
-                (0, 0, 0, cus + 1, 10), (0, 0, 0, 4, 0)):
+    for placement in range(1, 8):
+        r = probe.issue_cost(handle, 8, 24, True, cus, 500, placement=placement)
+        assert 1024 <= r["cycles_per_stage"] < 4 * 1024, (placement, r)
+    # without the matrix instructions the memory instructions show what they take by themselves;
+    # a DMA source larger than the vector L1 costs no less than one it holds
+    alone = probe.issue_cost(handle, 8, 24, True, cus, 500, mfma=False)
+    alone_l2 = probe.issue_cost(handle, 8, 24, True, cus, 500, mfma=False, src_kib_per_wave=32)
+    assert 0 < alone["cycles_per_stage"] < 4 * 1024 and 0 < alone_l2["cycles_per_stage"] < 8 * 1024
+    for bad in ((3, 0, 0, 0, 1, 8, 4, 10), (0, 12, 0, 0, 1, 8, 4, 10), (0, 0, 2, 0, 1, 8, 4, 10),
+                (0, 0, 0, 0, 1, 8, 0, 10), (0, 0, 0, 0, 1, 8, cus + 1, 10), (0, 0, 0, 0, 1, 8, 4, 0),
+                (8, 24, 1, 8, 1, 8, 4, 10), (4, 24, 1, 1, 1, 8, 4, 10), (8, 24, 1, 3, 0, 8, 4, 10),
+                (0, 0, 0, 0, 2, 8, 4, 10), (0, 0, 0, 0, 1, 4, 4, 10), (0, 0, 0, 0, 1, 2048, 4, 10)):
         assert lib.cigemm_probe_issue_cost(handle.raw, *bad, res) == Status.INVALID_VALUE
-    assert lib.cigemm_probe_issue_cost(handle.raw, 0, 0, 0, 4, 10, None) == Status.INVALID_VALUE
+    assert lib.cigemm_probe_issue_cost(handle.raw, 0, 0, 0, 0, 1, 8, 4, 10, None) == Status.INVALID_VALUE
+    # more DMA source than the handle's workspace holds: refused, nothing launched
+    assert lib.cigemm_probe_issue_cost(handle.raw, 8, 24, 1, 0, 1, 1024, cus, 10, res) == Status.NOT_SUPPORTED
