@@ -24,6 +24,10 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+# The CPU-baseline legs run the oracle's OpenMP loops in this process.  Worker threads that keep
+# spinning after a parallel region compete with the HIP runtime's own threads: the launch-bound
+# 512^3 call measured 8.9 us after such a leg and 5.9 us without.  Let them sleep instead.
+os.environ.setdefault("OMP_WAIT_POLICY", "passive")
 
 # MI355X published dense peaks: 256 CUs x 4 SIMDs x 2.4 GHz x 1024 flop/clk (16-bit), x2 for int8.
 PEAK_16BIT_TFLOPS = 2516.6
@@ -296,6 +300,56 @@ def decode_sweep(torch, ci, handle, steps, warmup):
     print(json.dumps({"decode_sweep": res}), flush=True)
 
 
+ONLY_WORKLOADS = ("bf16_8192", "fp16_8192", "int8_8192", "int8_8192_nk", "int8_4096_dequant_f32",
+                  "int8_linear_2048x11008x4096_dequant_bf16", "fp32_4096")
+
+
+def only_workload(torch, ci, wl, handle, name, steps, warmup):
+    """One of the matrix-core-bound workloads of the benchmark by itself (same inputs, same
+    protocol), for profiler runs whose statistics should cover one kernel: prints one JSON
+    object with its rate, time per call and kernel."""
+    if name in ("bf16_8192", "fp16_8192"):
+        kind = "bf16" if name.startswith("bf16") else "f16"
+        M = N = K = 8192
+        a_b, b_b = wl.normal_16bit(M, N, K, seed=2, kind=kind)
+        a, b = dev16(torch, a_b, kind), dev16(torch, b_b, kind)
+        c = torch.empty((M, N), dtype=a.dtype, device="cuda")
+        gemm = handle.gemm_bf16 if kind == "bf16" else handle.gemm_f16
+        fn, unit, peak = (lambda: gemm(a, b, out=c)), "TFLOP/s", PEAK_16BIT_TFLOPS
+    elif name in ("int8_8192", "int8_8192_nk"):
+        M = N = K = 8192
+        Aq, Bq, _, _ = wl.int8_uniform(M, N, K, seed=1)
+        nk = name.endswith("_nk")
+        a = torch.from_numpy(Aq).cuda()
+        b = torch.from_numpy(np.ascontiguousarray(Bq.T) if nk else Bq).cuda()
+        c = torch.empty((M, N), dtype=torch.int32, device="cuda")
+        fn, unit, peak = (lambda: handle.gemm_i8_i32(a, b, ci.B_NK if nk else ci.B_KN, out=c)), "TOP/s", PEAK_INT8_TOPS
+    elif name == "int8_4096_dequant_f32":
+        M = N = K = 4096
+        Aq, Bq, sa, sb = wl.int8_uniform(M, N, K, seed=1)
+        a, b, sa_d, sb_d = (torch.from_numpy(v).cuda() for v in (Aq, Bq, sa, sb))
+        c = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        fn, unit, peak = (lambda: handle.gemm_i8_dequant(a, b, sa_d, sb_d, ci.B_KN, ci.OUT_F32, out=c)), "TOP/s", PEAK_INT8_TOPS
+    elif name == "int8_linear_2048x11008x4096_dequant_bf16":
+        M, K, N = 2048, 4096, 11008
+        Xq, sx, Wq, sw = wl.quantized_linear(M, K, N, seed=3)
+        a, b, sa_d, sb_d = (torch.from_numpy(v).cuda() for v in (Xq, Wq, sx, sw))
+        c = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        fn, unit, peak = (lambda: handle.gemm_i8_dequant(a, b, sa_d, sb_d, ci.B_NK, ci.OUT_BF16, out=c)), "TOP/s", PEAK_INT8_TOPS
+    else:
+        M = N = K = 4096
+        Af, Bf = wl.fp32_uniform(M, N, K, seed=0)
+        a, b = torch.from_numpy(Af).cuda(), torch.from_numpy(Bf).cuda()
+        c = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        fn, unit, peak = (lambda: handle.gemm_f32(a, b, out=c)), "TFLOP/s", PEAK_FP32_MATRIX_TFLOPS
+    wall, ev = time_calls(torch, fn, steps, warmup)
+    ops = wl.gemm_ops(M, N, K)
+    rate = ops * steps / ev / 1e12
+    print(json.dumps({"only": name, "value": rate, "unit": unit, "frac_of_peak": rate / peak, "peak": peak,
+                      "ms": ev / steps * 1e3, "ms_wall": wall / steps * 1e3, "steps": steps, "warmup": warmup,
+                      "ops_per_call": ops, "kernel": handle.last_kernel}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -316,6 +370,8 @@ def main():
     ap.add_argument("--k-sweep", action="store_true",
                     help="instead of the benchmark: time the tile kernel at several K per M x N and "
                          "fit its fixed cost per tile and its cost per stage")
+    ap.add_argument("--only", choices=ONLY_WORKLOADS,
+                    help="instead of the benchmark: this one workload by itself (for profiler runs)")
     ap.add_argument("--decode-sweep", action="store_true",
                     help="instead of the benchmark: decode GEMMs (M = 1, 16, 32) at layer shapes of common "
                          "decoder models, bf16 and int8")
@@ -339,6 +395,9 @@ def main():
         return
     if args.decode_sweep:
         decode_sweep(torch, ci, handle, args.steps, args.warmup)
+        return
+    if args.only:
+        only_workload(torch, ci, wl, handle, args.only, args.steps, args.warmup)
         return
     n = args.size
     per_config = {}
@@ -797,18 +856,29 @@ def main():
         # instructions, the stage's 24 LDS fragment reads and its barrier added, all units busy.
         cus = torch.cuda.get_device_properties(0).multi_processor_count
         issue = {}
-        for n_dma, n_lds, bar in ((0, 0, 0), (2, 0, 0), (4, 0, 0), (8, 0, 0), (0, 24, 0), (0, 0, 1),
-                                  (8, 24, 0), (8, 24, 1)):
+
+        def ic(key, *a, **kw):
             for _ in range(2):
-                r_ic = probe.issue_cost(handle, n_dma, n_lds, bool(bar), cus, 4000)
-            issue[f"dma{n_dma}_lds{n_lds}_bar{bar}"] = round(r_ic["cycles_per_stage"], 1)
-        one = probe.issue_cost(handle, 8, 24, True, 1, 4000)
-        issue["dma8_lds24_bar1_one_workgroup"] = round(one["cycles_per_stage"], 1)
+                r_ic = probe.issue_cost(handle, *a, **kw)
+            issue[key] = round(r_ic["cycles_per_stage"], 1)
+
+        for n_dma, n_lds, bar in ((0, 0, 0), (8, 0, 0), (0, 24, 0), (0, 0, 1), (8, 24, 0)):
+            ic(f"dma{n_dma}_lds{n_lds}_bar{bar}", n_dma, n_lds, bool(bar), cus, 4000)
+        # all three, with the DMA instructions back to back after the barrier (placement 0) and in
+        # every second slot (placement 1, what the tile kernel does), sources the L1 holds or not
+        ic("dma8_lds24_bar1_back_to_back", 8, 24, True, cus, 4000)
+        ic("dma8_lds24_bar1_spread", 8, 24, True, cus, 4000, placement=1)
+        ic("dma8_lds24_bar1_spread_l2_source", 8, 24, True, cus, 4000, placement=1, src_kib_per_wave=32)
+        ic("dma8_lds24_bar1_spread_one_workgroup", 8, 24, True, 1, 4000, placement=1)
+        # the stage's memory instructions without its matrix instructions
+        ic("no_mfma_dma8", 8, 0, True, cus, 4000, mfma=False, placement=1, src_kib_per_wave=32)
+        ic("no_mfma_lds24", 0, 24, True, cus, 4000, mfma=False)
+        ic("no_mfma_dma8_lds24", 8, 24, True, cus, 4000, mfma=False, placement=1, src_kib_per_wave=32)
         mfma_probe["issue_cost_cycles_per_stage"] = issue
-        roofline["issue_ceiling"] = 1024.0 / issue["dma8_lds24_bar1"]
+        roofline["issue_ceiling"] = 1024.0 / issue["dma8_lds24_bar1_spread_l2_source"]
         roofline["issue_ceiling_what"] = ("1024 matrix-core issue cycles per stage / cycles per stage of a "
-                                          "register-resident loop with the stage's 8 LDS-DMA instructions, 24 "
-                                          "LDS fragment reads and barrier, same run")
+                                          "register-resident loop with the stage's 8 LDS-DMA instructions (every "
+                                          "second slot, L2 sources), 24 LDS fragment reads and barrier, same run")
         for k, v in per_config.items():
             log(f"[bench]   {k}: {json.dumps(v)}")
         log(f"[bench]   register-resident MFMA loop, T(FL)OP/s: {json.dumps(probe_res)}")

@@ -857,27 +857,47 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   const int steady_end = (pair_valid < 8 && !(KTS & 1)) ? KTS - 2 : KTS;
   typedef std::integral_constant<int, -1> any_phase_t;
   int s = 0;
-  // twelve stages at a time with every ring slot a constant (the slot variables keep their
-  // values of phase 0 meanwhile: s stays a multiple of 12) ...
-  for (; s + 11 + 5 < steady_end; s += 12) {
-    stage(s, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 0>{});
-    stage(s + 1, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 1>{});
-    stage(s + 2, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 2>{});
-    stage(s + 3, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 3>{});
-    stage(s + 4, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 4>{});
-    stage(s + 5, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 5>{});
-    stage(s + 6, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 6>{});
-    stage(s + 7, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 7>{});
-    stage(s + 8, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 8>{});
-    stage(s + 9, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 9>{});
-    stage(s + 10, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, 10>{});
-    stage(s + 11, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, 11>{});
+  // The steady part, in stage pairs (s, s + 1) with s + 5 < steady_end, every ring slot a
+  // constant: whole trips of twelve stages, then up to five more pairs as straight-line code
+  // whose phases go on from 0 (s is a multiple of 12 there).  The slot variables are not kept up
+  // to date meanwhile.
+#define CIG_STEADY_PAIR(P)                                                                      \
+  stage(s, std::integral_constant<int, 0>{}, steady_t{}, std::integral_constant<int, P>{});     \
+  stage(s + 1, std::integral_constant<int, 1>{}, steady_t{}, std::integral_constant<int, P + 1>{}); \
+  s += 2;
+  const int steady_pairs = steady_end > 5 ? (steady_end - 4) / 2 : 0;
+  const int rest_pairs = steady_pairs % 6;
+  for (int trip = steady_pairs / 6; trip > 0; --trip) {
+    CIG_STEADY_PAIR(0)
+    CIG_STEADY_PAIR(2)
+    CIG_STEADY_PAIR(4)
+    CIG_STEADY_PAIR(6)
+    CIG_STEADY_PAIR(8)
+    CIG_STEADY_PAIR(10)
   }
-  // ... then the rest of the steady part and the drain, with the slots advanced at run time
-  for (; s + 5 < steady_end; s += 2) {
-    stage(s, std::integral_constant<int, 0>{}, steady_t{}, any_phase_t{});
-    stage(s + 1, std::integral_constant<int, 1>{}, steady_t{}, any_phase_t{});
+  if (rest_pairs > 0) {
+    CIG_STEADY_PAIR(0)
+    if (rest_pairs > 1) {
+      CIG_STEADY_PAIR(2)
+      if (rest_pairs > 2) {
+        CIG_STEADY_PAIR(4)
+        if (rest_pairs > 3) {
+          CIG_STEADY_PAIR(6)
+          if (rest_pairs > 4) {
+            CIG_STEADY_PAIR(8)
+          }
+        }
+      }
+    }
   }
+#undef CIG_STEADY_PAIR
+  // ... then the drain, whose stages advance the slots at run time, from the slots of stage s
+  slot = BPAIR ? (s / 2) % 2 : s % NSTAGES;
+  next_slot = BPAIR ? 1 - slot : (s + 1) % NSTAGES;
+  dma_slot = (s + DIST) % NSTAGES;
+  pslot = (s / 2) % 3;
+  next_pslot = (s / 2 + 1) % 3;
+  dma_pslot = (s / 2 + 2) % 3;
   for (; s + 1 < KTS; s += 2) {
     stage(s, std::integral_constant<int, 0>{}, drain_t{}, any_phase_t{});
     stage(s + 1, std::integral_constant<int, 1>{}, drain_t{}, any_phase_t{});
@@ -1052,33 +1072,23 @@ struct epi_register_heavy<E, typename std::enable_if<E::REGISTER_HEAVY>::type> :
 
 // The 256-row tile has two forms that fetch, multiply and store the same data in the same
 // order (results identical bit for bit): four waves of 128 x 128, one per SIMD, and eight waves
-// of 64 x 128, two per SIMD, where one wave's DMA issue hides under the other's MFMAs at 1.5 x
-// the LDS fragment traffic.  The second takes 7 % fewer cycles, but in sustained runs the
-// chip is power limited and answers with a lower clock: bf16 on N(0,1) data -0.5 % in time,
-// int8 K x N +-0.4 %, int8 N x K +1.4..2.1 % (200 launches each, alternating, one box; +1..4 %
-// everywhere in short runs on low-entropy data), fp32 +0.2 % (its MFMA shares the vector ALU).
-// With one round of tiles (4096^3: 256 tiles, 1000 launches on N(0,1) data) bf16 gains 1.9 %,
-// int8 K x N loses 2 %.  So N x K int8 weights use it always, the 16-bit types when the tiles
-// fit one round.
+// of 64 x 128, two per SIMD, where one wave's other instructions issue under the other's MFMAs,
+// at 1.5 x the LDS fragment traffic.  Since the four-wave main loop carries no ring arithmetic
+// (12-stage body, see `stage`) the second form has little left to hide, and the chip, power
+// limited, answers its extra LDS traffic with a lower clock.  Alternating in one process on the
+// bench's data: bf16 8192^3 -0.1..+0.3 % for four waves, int8 N x K 8192^3 +-0.3 %, bf16 4096^3
+// (one round) +1.1 %, int8 N x K 4096^3 -> int32 +6.8 %; only N x K int8 weights with a 16-bit
+// output keep the eight waves (2048 x 11008 x 4096 at M = 1024, one round: 44.0 against 44.8 us).
 template <typename Math, int BMODE, typename Epi>
 void launch_tile_256(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
                      int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi,
                      int splits = 1) {
-  if constexpr (BMODE == B_NK && !epi_register_heavy<Epi>::value) {
+  if constexpr (BMODE == B_NK && Epi::OUT_BYTES == 2 && !epi_register_heavy<Epi>::value)
     launch_tile_mt<Math, BMODE, 2, Epi, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi,
                                            splits);
-  } else {
-    if constexpr (Math::ELEM_BYTES == 2 && !epi_register_heavy<Epi>::value) {
-      const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-      if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) * splits <= cus) {
-        launch_tile_mt<Math, BMODE, 2, Epi, 4>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes,
-                                               epi, splits);
-        return;
-      }
-    }
+  else
     launch_tile_mt<Math, BMODE, 4, Epi, 2>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi,
                                            splits);
-  }
 }
 
 // The 128-row tile has the same two forms (four waves of 64 x 128, eight of 32 x 128); with

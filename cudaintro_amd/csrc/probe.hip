@@ -216,6 +216,14 @@ __global__ __launch_bounds__(256, 1) void issue_cost_kernel(const char* __restri
         mfma_piece(f0, sl);
         if (NLDS && sl < 12) read_piece(f1, 1, sl);
         if (dma_in_slot(16 + sl, OFF, STRIDE, NDMA)) dma(dma_index(16 + sl, OFF, STRIDE, NDMA));
+        if (sl == 13) {
+          // the next stage's DMA source, computed here, in a slot that holds nothing else (a
+          // lone wave issues one instruction per four cycles, and only about seven of them fit
+          // under one matrix instruction: at the end of the loop, beside the branch, these few
+          // scalar instructions would cost 24 cycles per stage)
+          src_off = src_off + 8192 < src_span ? src_off + 8192 : 0;
+          my_src = my_src0 + src_off;
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
       // (as in the product: everything but the DMA of the last two stages has landed)
@@ -231,8 +239,6 @@ __global__ __launch_bounds__(256, 1) void issue_cost_kernel(const char* __restri
         __builtin_amdgcn_sched_barrier(0);
       }
       asm volatile("" ::: "memory");
-      src_off = src_off + 8192 < src_span ? src_off + 8192 : 0;
-      my_src = my_src0 + src_off;
     }
   };
   if (WOFF == 0 || w == 0)
