@@ -591,12 +591,12 @@ def main():
             t = wl.gemm_ops(M, N, K) * args.steps / e / 1e12
             per_config[name] = {"tops": t, "frac_of_peak": t / PEAK_INT8_TOPS, "peak": PEAK_INT8_TOPS,
                                 "ms": e / args.steps * 1e3, "kernel": handle.last_kernel}
-            if lay == ci.B_KN:
+            if lay == ci.B_KN or "192x256" in handle.last_kernel:
                 # phases of the same tile kernel with raw int32 output (the same bytes per
                 # output element as the fp32 dequantized one)
                 o32 = out if not dequant else torch.empty((M, N), dtype=torch.int32, device="cuda")
                 for _ in range(3):
-                    ph = probe.tile_phases(handle, a, b, o32)
+                    ph = probe.tile_phases(handle, a, b, o32, b_nk=lay == ci.B_NK)
                 per_config[name]["phases_raw_i32_out"] = ph
                 del o32
             if not args.no_cpu:
@@ -929,6 +929,10 @@ def main():
     }
     # the metric's three dtypes, flat (beside roofline.per_dtype)
     for dt, rec in per_dtype.items():
+        pkey = f"{dt}_{n}"
+        if f"{pkey}_mfma_busy" in prof:
+            rec["from_profiles"] = {"mfma_busy": prof[f"{pkey}_mfma_busy"], "clock_ghz": prof[f"{pkey}_clock_ghz"],
+                                    "traffic": prof.get(pkey)}
         unit = "tflops" if dt != "int8" else "tops"
         line[f"{dt}_{n}_{unit}"] = rec["achieved"]
         line[f"{dt}_{n}_frac_of_peak"] = rec["frac"]

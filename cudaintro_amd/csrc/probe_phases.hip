@@ -13,11 +13,11 @@
 namespace cig {
 namespace {
 
-template <typename Math, int BMODE, bool TWO_PER_UNIT, typename Epi>
+template <typename Math, int BMODE, bool TWO_PER_UNIT, typename Epi, int MT = 4>
 cigemmStatus_t run_profiled(cigemmContext* ctx, const char* name, int64_t M, int64_t N,
                             int64_t K_bytes, const void* A, int64_t lda_bytes, const void* B,
                             int64_t ldb_bytes, const Epi& base, double* out) {
-  constexpr int ROWS = TWO_PER_UNIT ? tile::T2_TILE_M : 256;
+  constexpr int ROWS = TWO_PER_UNIT ? tile::T2_TILE_M : 64 * MT;
   const int64_t tiles = ((M + ROWS - 1) / ROWS) * ((N + tile::BN - 1) / tile::BN);
   if (!ctx->workspace || (size_t)tiles * 64 > ctx->ws_partial_bytes)
     return fail(ctx, CIGEMM_STATUS_NOT_SUPPORTED, "%s: %lld tiles exceed the workspace", name,
@@ -28,8 +28,8 @@ cigemmStatus_t run_profiled(cigemmContext* ctx, const char* name, int64_t M, int
     tile::launch_tile2<Math, BMODE, tile::EpiProfiled<Epi>>(ctx, M, N, K_bytes, A, lda_bytes, B,
                                                             ldb_bytes, epi);
   else
-    tile::launch_tile_mt<Math, BMODE, 4, tile::EpiProfiled<Epi>, 2>(ctx, M, N, K_bytes, A,
-                                                                   lda_bytes, B, ldb_bytes, epi);
+    tile::launch_tile_mt<Math, BMODE, MT, tile::EpiProfiled<Epi>, 2>(ctx, M, N, K_bytes, A,
+                                                                    lda_bytes, B, ldb_bytes, epi);
   cigemmStatus_t st = check_launch(ctx, name);
   if (st != CIGEMM_STATUS_SUCCESS) return st;
   std::vector<uint64_t> h((size_t)tiles * 8);
@@ -85,11 +85,11 @@ extern "C" cigemmStatus_t cigemm_probe_tile_phases(cigemmHandle_t h, int kind, i
                                                    void* C, int64_t ldc, double* phases) {
   const char* name = "cigemm_probe_tile_phases";
   if (!h || h->magic != kCtxMagic) return CIGEMM_STATUS_NOT_INITIALIZED;
-  if (kind < 0 || kind > 4 || !A || !B || !C || !phases || M <= 0 || N <= 0 || K <= 0 ||
-      lda < K || ldb < N || ldc < N)
+  if (kind < 0 || kind > 5 || !A || !B || !C || !phases || M <= 0 || N <= 0 || K <= 0 ||
+      lda < K || ldb < (kind == 5 ? K : N) || ldc < N)
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: bad argument", name);
-  const int elem = (kind == 1 || kind == 3) ? 1 : 2;
-  if (!tile::tile_shape_ok(M, N, K, elem, A, lda, B, ldb, true) || N % 8 || ldc % 8 ||
+  const int elem = (kind == 1 || kind == 3 || kind == 5) ? 1 : 2;
+  if (!tile::tile_shape_ok(M, N, K, elem, A, lda, B, ldb, kind != 5) || N % 8 || ldc % 8 ||
       ((uintptr_t)C & 15))
     return fail(h, CIGEMM_STATUS_NOT_SUPPORTED, "%s: shape or alignment outside the tile kernel's",
                 name);
@@ -97,6 +97,9 @@ extern "C" cigemmStatus_t cigemm_probe_tile_phases(cigemmHandle_t h, int kind, i
   const EpiStoreI32x4 e32{static_cast<int32_t*>(C), ldc};
   const EpiStore16x4<F16> e16h{static_cast<uint16_t*>(C), ldc};
   switch (kind) {
+    case 5:
+      return run_profiled<tile::MathI8, tile::B_NK, false, EpiStoreI32x4, 3>(h, name, M, N, K, A, lda, B,
+                                                                            ldb, e32, phases);
     case 4:
       return run_profiled<tile::MathF16, tile::B_KN16, false>(h, name, M, N, K * 2, A, lda * 2, B,
                                                               ldb * 2, e16h, phases);

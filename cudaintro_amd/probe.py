@@ -81,17 +81,21 @@ PHASE_KEYS = ("prologue_us", "main_loop_us", "epilogue_us", "first_start_to_last
               "cycles_per_stage", "main_loop_clock_ghz", "first_epilogue_to_last_end_us", "workgroups")
 
 
-def tile_phases(h: Handle, A, B, out, paired=False):
+def tile_phases(h: Handle, A, B, out, paired=False, b_nk=False):
     """One instrumented launch of the 256-row tile kernel (bf16, fp16 or int8 K x N -> int32), or
-    with ``paired`` of its two-workgroups-per-unit form (bf16, int8); the phase figures as a dict."""
+    with ``paired`` of its two-workgroups-per-unit form (bf16, int8), or with ``b_nk`` of the
+    192-row kernel over int8 N x K weights; the phase figures as a dict."""
     import torch
-    if A.dtype == torch.float16:
+    if b_nk:
+        assert A.dtype == torch.int8 and not paired
+        kind = 5
+    elif A.dtype == torch.float16:
         assert not paired
         kind = 4
     else:
         kind = {torch.bfloat16: 0, torch.int8: 1}[A.dtype] + (2 if paired else 0)
     M, K = A.shape
-    N = B.shape[1]
+    N = B.shape[0] if b_nk else B.shape[1]
     ph = (C.c_double * 8)()
     st = load_library().cigemm_probe_tile_phases(h.raw, kind, M, N, K, A.data_ptr(), Handle._ld(A),
                                                  B.data_ptr(), Handle._ld(B), out.data_ptr(),

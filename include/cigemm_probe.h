@@ -66,7 +66,9 @@ CIGEMM_API cigemmStatus_t cigemm_probe_issue_cost(cigemmHandle_t handle, int n_d
  * the stamps: kind 0 = bf16 (A, B, C as in cigemm_gemm_bf16), 1 = int8 K x N operands, int32
  * out (as cigemm_gemm_i8_i32 with CIGEMM_B_KN); 2 and 3 = the same two on the
  * two-workgroups-per-unit form of the kernel (128-row tiles; "stage" then means a stage of
- * such a tile, 512 matrix-core issue cycles instead of 1024); 4 = fp16 (as cigemm_gemm_f16).
+ * such a tile, 512 matrix-core issue cycles instead of 1024); 4 = fp16 (as cigemm_gemm_f16);
+ * 5 = int8 with N x K weights on 192-row tiles, int32 out (as cigemm_gemm_i8_i32 with
+ * CIGEMM_B_NK; the form the quantized linear-layer shape runs on: 768 issue cycles per stage).
  * Same shape and alignment conditions as the tile kernel, N % 8 == 0.
  * phases[0..7] receive, averaged over the workgroups: microseconds from workgroup start to the
  * first stage in registers; of the main loop; of the epilogue until its stores are

@@ -49,6 +49,20 @@ def test_probe_output_equals_plain_call_and_phases_add_up(handle, torch_gpu, ora
         assert 0.05 < ph["main_loop_clock_ghz"] < 3.0
 
 
+def test_probe_nk_192_row_form(handle, torch_gpu, rng):
+    """kind 5: the 192-row kernel over N x K int8 weights gives the library's bits."""
+    torch = torch_gpu
+    M, N, K = 600, 520, 1040
+    a = torch.from_numpy(rng.integers(-127, 128, size=(M, K), dtype=np.int8)).cuda()
+    b = torch.from_numpy(rng.integers(-127, 128, size=(N, K), dtype=np.int8)).cuda()
+    with handle.algo(ci.ALGO_TILE):
+        want = handle.gemm_i8_i32(a, b, ci.B_NK)
+    out = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    ph = probe.tile_phases(handle, a, b, out, b_nk=True)
+    assert torch.equal(out, want)
+    assert ph["workgroups"] == -(-M // 192) * -(-N // 256) and ph["cycles_per_stage"] >= 768
+
+
 def test_probe_rejects_bad_arguments(handle, torch_gpu):
     torch = torch_gpu
     a = torch.zeros((64, 60), dtype=torch.bfloat16, device="cuda")      # K * 2 not a multiple of 16
