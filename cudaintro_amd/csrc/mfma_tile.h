@@ -1,8 +1,8 @@
 // The LDS-tiled MFMA GEMM kernel shared by the bf16, fp16 and int8 families.
 //
-// Workgroup = 256 lanes = 4 waves (2 x 2) -- or, for the 256- and 128-row tiles over N x K int8
-// weights, 512 lanes = 8 waves (4 x 2) of half the height, two per SIMD, same data flow, see
-// launch_tile_256 / launch_tile_128 --; macro tile 256 (m) x 256 (n); k is consumed in
+// Workgroup = 256 lanes = 4 waves (2 x 2) -- or, for N x K int8 weights with a 16-bit output and
+// for their 128-row tiles, 512 lanes = 8 waves (4 x 2) of half the height, two per SIMD, same data
+// flow, see launch_tile_256 / launch_tile_128 --; macro tile 256 (m) x 256 (n); k is consumed in
 // stages of 64 BYTES per row (32 halves, 64 int8 or 16 floats) = two MFMA k-steps.  Each wave
 // owns a 128 x 128 block = 4 x 4 MFMA tiles of 32 x 32 = 256 accumulators per lane (the AGPR
 // file); one wave per SIMD.  The tile height is a template parameter (MT = 4, 3, 2 or 1 row
@@ -37,7 +37,8 @@
 // Pipeline, iteration s (B of stage s sits in slot s % 4, A in pair slot (s / 2) % 3):
 //   k-step 0: 16 MFMAs on the fragments of (s,0); under them the 12 LDS reads of (s,1)
 //   wait until this wave's DMA of stage s+1 has landed (vmcnt), workgroup barrier
-//   k-step 1: 16 MFMAs on (s,1); under them the 12 LDS reads of (s+1,0) and the DMA:
+//   k-step 1: 16 MFMAs on (s,1); under them the 12 LDS reads of (s+1,0) and the DMA, one
+//             instruction in every second MFMA slot:
 //             4 instructions of B of stage s+3 into the slot stage s-1 just left (every wave
 //             finished reading it before it reached the barrier) and 4 of the 8 of an A
 //             pair: the first half of the pair of stages s+4, s+5 when s is even, the second
@@ -46,7 +47,10 @@
 // s+5, odd stages the B pair of stages s+3, s+4 (into the slot whose last fragments were read
 // in k-step 0 of that stage).
 // Fragments are double buffered in registers.  The emitted order is pinned slot by slot
-// with scheduling fences: one MFMA, at most one LDS read, at most one DMA.
+// with scheduling fences: one MFMA, at most one LDS read, at most one DMA.  The ring slots
+// repeat every 12 stages (4 B slots, 3 A pair slots of 2 stages): the steady part of the main
+// loop runs in trips of 12 stages whose slots are all compile-time constants, so that no ring
+// or address arithmetic is left between the matrix instructions (see `stage` below).
 //
 // The MFMA is issued with the B fragment as its first operand and the A fragment as its
 // second, so it yields the transposed 32 x 32 block: lane l holds, for the single output
