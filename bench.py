@@ -437,6 +437,16 @@ def main():
     roofline["mfma_issue_fraction_of_main_loop"] = 1024.0 / phases["cycles_per_stage"]
     roofline["median_kernel_ms"] = median_call_ms(torch, lambda: handle.gemm_bf16(A, B, out=C),
                                                   max(50, args.steps))
+    # What the 4.3 x re-read operand traffic costs: the same instrumented launch with every
+    # workgroup on output tile (0, 0), so that no operand read leaves the L2.
+    for _ in range(3):
+        ph_l2 = probe.tile_phases(handle, A, B, C, same_tile=True)
+    roofline["all_operands_in_l2"] = {
+        "launch_us": ph_l2["first_start_to_last_end_us"], "launch_us_real_tiles": phases["first_start_to_last_end_us"],
+        "main_loop_us": ph_l2["main_loop_us"], "cycles_per_stage": ph_l2["cycles_per_stage"],
+        "clock_ghz": ph_l2["main_loop_clock_ghz"],
+        "what": "one instrumented launch with every workgroup computing output tile (0, 0)"}
+    handle.gemm_bf16(A, B, out=C)
     # HBM-side bytes per launch and the counter decomposition of the same kernel are not
     # measurable from inside this process: they come from the rocprofv3 --pmc runs of this
     # same command summarised in profiles/ (the file says which runs).  Everything copied from

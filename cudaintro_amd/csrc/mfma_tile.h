@@ -365,6 +365,10 @@ struct epi_profiled<E, typename std::enable_if<E::PROFILED>::type> : std::true_t
 template <typename Epi>
 struct EpiProfiled : Epi {
   uint64_t* stamps;
+  // Non-zero: every workgroup computes output tile (0, 0) instead of its own (all of them read
+  // the same two operand panels, which then stay in every L2, and store the same values to the
+  // same place): what the launch would take if no operand read ever left the L2.
+  int same_tile;
   static constexpr bool PROFILED = true;
 };
 
@@ -550,6 +554,9 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
   // so that everything derived from them, the DMA base addresses above all, stays scalar)
   tm = __builtin_amdgcn_readfirstlane(tm);
   tn = __builtin_amdgcn_readfirstlane(tn);
+  if constexpr (epi_profiled<Epi>::value) {
+    if (epi.same_tile) tm = tn = 0;
+  }
   const int64_t m0 = (int64_t)tm * TILE_M, n0 = (int64_t)tn * BN;
   // Per-tensor operands of the epilogue: one word each at a uniform address, read here, before
   // anything is written, hence with a scalar load whose latency nothing waits for.

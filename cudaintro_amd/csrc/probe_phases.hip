@@ -16,14 +16,14 @@ namespace {
 template <typename Math, int BMODE, bool TWO_PER_UNIT, typename Epi, int MT = 4>
 cigemmStatus_t run_profiled(cigemmContext* ctx, const char* name, int64_t M, int64_t N,
                             int64_t K_bytes, const void* A, int64_t lda_bytes, const void* B,
-                            int64_t ldb_bytes, const Epi& base, double* out) {
+                            int64_t ldb_bytes, const Epi& base, double* out, int same_tile = 0) {
   constexpr int ROWS = TWO_PER_UNIT ? tile::T2_TILE_M : 64 * MT;
   const int64_t tiles = ((M + ROWS - 1) / ROWS) * ((N + tile::BN - 1) / tile::BN);
   if (!ctx->workspace || (size_t)tiles * 64 > ctx->ws_partial_bytes)
     return fail(ctx, CIGEMM_STATUS_NOT_SUPPORTED, "%s: %lld tiles exceed the workspace", name,
                 (long long)tiles);
   uint64_t* stamps = static_cast<uint64_t*>(ctx->workspace);
-  tile::EpiProfiled<Epi> epi{base, stamps};
+  tile::EpiProfiled<Epi> epi{base, stamps, same_tile};
   if constexpr (TWO_PER_UNIT)
     tile::launch_tile2<Math, BMODE, tile::EpiProfiled<Epi>>(ctx, M, N, K_bytes, A, lda_bytes, B,
                                                             ldb_bytes, epi);
@@ -85,6 +85,9 @@ extern "C" cigemmStatus_t cigemm_probe_tile_phases(cigemmHandle_t h, int kind, i
                                                    void* C, int64_t ldc, double* phases) {
   const char* name = "cigemm_probe_tile_phases";
   if (!h || h->magic != kCtxMagic) return CIGEMM_STATUS_NOT_INITIALIZED;
+  // kind + 16: kinds 0, 1 and 4 with every workgroup on output tile (0, 0)
+  const int same_tile = (kind == 16 || kind == 17 || kind == 20) ? 1 : 0;
+  if (same_tile) kind -= 16;
   if (kind < 0 || kind > 5 || !A || !B || !C || !phases || M <= 0 || N <= 0 || K <= 0 ||
       lda < K || ldb < (kind == 5 ? K : N) || ldc < N)
     return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: bad argument", name);
@@ -102,13 +105,13 @@ extern "C" cigemmStatus_t cigemm_probe_tile_phases(cigemmHandle_t h, int kind, i
                                                                             ldb, e32, phases);
     case 4:
       return run_profiled<tile::MathF16, tile::B_KN16, false>(h, name, M, N, K * 2, A, lda * 2, B,
-                                                              ldb * 2, e16h, phases);
+                                                              ldb * 2, e16h, phases, same_tile);
     case 0:
       return run_profiled<tile::MathBF16, tile::B_KN16, false>(h, name, M, N, K * 2, A, lda * 2, B,
-                                                               ldb * 2, e16, phases);
+                                                               ldb * 2, e16, phases, same_tile);
     case 1:
       return run_profiled<tile::MathI8, tile::B_KN8, false>(h, name, M, N, K, A, lda, B, ldb, e32,
-                                                            phases);
+                                                            phases, same_tile);
     case 2:
       return run_profiled<tile::MathBF16, tile::B_KN16, true>(h, name, M, N, K * 2, A, lda * 2, B,
                                                               ldb * 2, e16, phases);

@@ -81,7 +81,7 @@ PHASE_KEYS = ("prologue_us", "main_loop_us", "epilogue_us", "first_start_to_last
               "cycles_per_stage", "main_loop_clock_ghz", "first_epilogue_to_last_end_us", "workgroups")
 
 
-def tile_phases(h: Handle, A, B, out, paired=False, b_nk=False):
+def tile_phases(h: Handle, A, B, out, paired=False, b_nk=False, same_tile=False):
     """One instrumented launch of the 256-row tile kernel (bf16, fp16 or int8 K x N -> int32), or
     with ``paired`` of its two-workgroups-per-unit form (bf16, int8), or with ``b_nk`` of the
     192-row kernel over int8 N x K weights; the phase figures as a dict."""
@@ -94,6 +94,9 @@ def tile_phases(h: Handle, A, B, out, paired=False, b_nk=False):
         kind = 4
     else:
         kind = {torch.bfloat16: 0, torch.int8: 1}[A.dtype] + (2 if paired else 0)
+    if same_tile:
+        assert kind in (0, 1, 4)
+        kind += 16
     M, K = A.shape
     N = B.shape[0] if b_nk else B.shape[1]
     ph = (C.c_double * 8)()

@@ -69,6 +69,10 @@ CIGEMM_API cigemmStatus_t cigemm_probe_issue_cost(cigemmHandle_t handle, int n_d
  * such a tile, 512 matrix-core issue cycles instead of 1024); 4 = fp16 (as cigemm_gemm_f16);
  * 5 = int8 with N x K weights on 192-row tiles, int32 out (as cigemm_gemm_i8_i32 with
  * CIGEMM_B_NK; the form the quantized linear-layer shape runs on: 768 issue cycles per stage).
+ * kind + 16 (kinds 0, 1 and 4 only): the same launch with every workgroup computing output
+ * tile (0, 0) -- all read the same two operand panels, which stay in every L2, and store the same
+ * values to the same place -- i.e. what the launch takes when no operand read leaves the L2 (C
+ * then holds the right values in its first tile only).
  * Same shape and alignment conditions as the tile kernel, N % 8 == 0.
  * phases[0..7] receive, averaged over the workgroups: microseconds from workgroup start to the
  * first stage in registers; of the main loop; of the epilogue until its stores are

@@ -49,6 +49,21 @@ def test_probe_output_equals_plain_call_and_phases_add_up(handle, torch_gpu, ora
         assert 0.05 < ph["main_loop_clock_ghz"] < 3.0
 
 
+def test_probe_same_tile_mode(handle, torch_gpu, oracle, rng):
+    """kind + 16: every workgroup computes tile (0, 0); that tile of the output is right."""
+    torch = torch_gpu
+    M, N, K = 768, 1024, 512
+    a = torch.from_numpy(rng.integers(-127, 128, size=(M, K), dtype=np.int8)).cuda()
+    b = torch.from_numpy(rng.integers(-127, 128, size=(K, N), dtype=np.int8)).cuda()
+    with handle.algo(ci.ALGO_TILE):
+        want = handle.gemm_i8_i32(a, b, ci.B_KN)
+    out = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    ph = probe.tile_phases(handle, a, b, out, same_tile=True)
+    assert ph["workgroups"] == 12
+    assert torch.equal(out[:256, :256], want[:256, :256])
+    assert not out[256:].any() and not out[:, 256:].any()
+
+
 def test_probe_nk_192_row_form(handle, torch_gpu, rng):
     """kind 5: the 192-row kernel over N x K int8 weights gives the library's bits."""
     torch = torch_gpu
