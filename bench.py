@@ -431,6 +431,10 @@ def main():
     for _ in range(3):
         phases = probe.tile_phases(handle, A, B, C)
     roofline["phases"] = phases
+    # every compute die holds its own clock and gets the same number of tiles: the launch ends
+    # with the slowest die, the average unit earlier
+    roofline["xcd_clock_ghz_slowest_fastest"] = [phases["slowest_xcd_clock_ghz"], phases["fastest_xcd_clock_ghz"]]
+    roofline["mean_unit_end_over_launch_end"] = phases["mean_unit_end_us"] / phases["first_start_to_last_end_us"]
     roofline["clock_ghz_main_loop_this_run"] = phases["main_loop_clock_ghz"]
     # matrix-core issue cycles of one 64-byte stage of the 256 x 256 tile: 32 instructions of 8
     # passes of 4 cycles per wave

@@ -357,7 +357,8 @@ struct epi_has_uniform_mode<E, typename std::enable_if<E::HAS_UNIFORM_MODE>::typ
 // Measurement aid: an epilogue that declares `static constexpr bool PROFILED = true` and carries
 // `uint64_t* stamps` makes the kernel record, per workgroup, the shader-clock counter and the
 // constant-rate counter at four points: start, first stage landed, main loop done, epilogue done
-// (stamps[8 * workgroup + 2 * point + {0, 1}]).
+// (stamps[8 * workgroup + 2 * point + {0, 1}]; at the first point the hardware id of the unit
+// the workgroup runs on takes the place of the shader-clock count).
 template <typename E, typename = void>
 struct epi_profiled : std::false_type {};
 template <typename E>
@@ -541,7 +542,11 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
     if constexpr (epi_profiled<Epi>::value) {
       if (threadIdx.x == 0) {
         uint64_t* p = epi.stamps + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 8 + 2 * point;
-        p[0] = __builtin_amdgcn_s_memtime();
+        // (point 0 carries, in place of the shader-clock count nobody reads there, where the
+        // workgroup runs: HW_ID in the low word, XCC_ID above it)
+        p[0] = point == 0 ? ((uint64_t)__builtin_amdgcn_s_getreg((3 << 11) | 20) << 32) |
+                                __builtin_amdgcn_s_getreg((31 << 11) | 4)
+                          : __builtin_amdgcn_s_memtime();
         p[1] = __builtin_amdgcn_s_memrealtime();
       }
     }

@@ -60,7 +60,9 @@ __global__ __launch_bounds__(256, 2) void mfma_tile2_kernel(int M, int N, int ti
     if constexpr (epi_profiled<Epi>::value) {
       if (threadIdx.x == 0) {
         uint64_t* p = epi.stamps + (int64_t)blockIdx.x * 8 + 2 * point;
-        p[0] = __builtin_amdgcn_s_memtime();
+        p[0] = point == 0 ? ((uint64_t)__builtin_amdgcn_s_getreg((3 << 11) | 20) << 32) |
+                                __builtin_amdgcn_s_getreg((31 << 11) | 4)
+                          : __builtin_amdgcn_s_memtime();
         p[1] = __builtin_amdgcn_s_memrealtime();
       }
     }

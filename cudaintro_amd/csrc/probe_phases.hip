@@ -4,6 +4,7 @@
 // per stage and the shader clock the chip held in the main loop.  The kernel is the product
 // kernel itself (same template, same schedule); only the four stamps are added.
 #include <algorithm>
+#include <utility>
 #include <vector>
 
 #include "cigemm_probe.h"
@@ -70,6 +71,43 @@ cigemmStatus_t run_profiled(cigemmContext* ctx, const char* name, int64_t M, int
   out[5] = main_ticks > 0 ? main_cycles / (main_ticks * tick_us) * 1e-3 : 0.0;
   out[6] = (double)(last_end - first_epi) * tick_us;  // first epilogue start -> last end
   out[7] = (double)tiles;
+  // Per XCD (the chip's eight compute dies hold their own clocks): main-loop clock of the
+  // slowest and of the fastest die; and per compute unit the end of its last workgroup, averaged
+  // over the units: the launch ends with the slowest unit, `out[3]`.
+  {
+    double xcc_cycles[16] = {0}, xcc_ticks[16] = {0};
+    std::vector<std::pair<uint64_t, uint64_t>> unit_end;  // (unit key, end of its last workgroup)
+    for (int64_t g = 0; g < tiles; ++g) {
+      const uint64_t* s = &h[(size_t)g * 8];
+      const int xcc = (int)((s[0] >> 32) & 15);
+      xcc_cycles[xcc] += (double)(s[4] - s[2]);
+      xcc_ticks[xcc] += (double)(s[5] - s[3]);
+      // unit = (XCC, shader engine, shader array, compute unit) of the hardware id
+      const uint64_t key = ((s[0] >> 32) << 16) | ((s[0] >> 8) & 0xff);
+      unit_end.emplace_back(key, s[7]);
+    }
+    double lo = 0, hi = 0;
+    int dies = 0;
+    for (int x = 0; x < 16; ++x)
+      if (xcc_ticks[x] > 0) {
+        const double ghz = xcc_cycles[x] / (xcc_ticks[x] * tick_us) * 1e-3;
+        lo = dies ? std::min(lo, ghz) : ghz;
+        hi = dies ? std::max(hi, ghz) : ghz;
+        ++dies;
+      }
+    std::sort(unit_end.begin(), unit_end.end());
+    double sum_end = 0;
+    int units = 0;
+    for (size_t i = 0; i < unit_end.size(); ++i)
+      if (i + 1 == unit_end.size() || unit_end[i + 1].first != unit_end[i].first) {
+        sum_end += (double)(unit_end[i].second - first_start) * tick_us;
+        ++units;
+      }
+    out[8] = lo;
+    out[9] = hi;
+    out[10] = units ? sum_end / units : 0.0;
+    out[11] = (double)units;
+  }
   ctx->last_kernel = "tile_phase_probe";
   return CIGEMM_STATUS_SUCCESS;
 }

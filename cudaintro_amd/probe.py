@@ -78,7 +78,8 @@ def issue_cost(h: Handle, n_dma: int, n_lds_reads: int, barrier: bool, workgroup
 
 
 PHASE_KEYS = ("prologue_us", "main_loop_us", "epilogue_us", "first_start_to_last_end_us",
-              "cycles_per_stage", "main_loop_clock_ghz", "first_epilogue_to_last_end_us", "workgroups")
+              "cycles_per_stage", "main_loop_clock_ghz", "first_epilogue_to_last_end_us", "workgroups",
+              "slowest_xcd_clock_ghz", "fastest_xcd_clock_ghz", "mean_unit_end_us", "units")
 
 
 def tile_phases(h: Handle, A, B, out, paired=False, b_nk=False, same_tile=False):
@@ -99,7 +100,7 @@ def tile_phases(h: Handle, A, B, out, paired=False, b_nk=False, same_tile=False)
         kind += 16
     M, K = A.shape
     N = B.shape[0] if b_nk else B.shape[1]
-    ph = (C.c_double * 8)()
+    ph = (C.c_double * 12)()
     st = load_library().cigemm_probe_tile_phases(h.raw, kind, M, N, K, A.data_ptr(), Handle._ld(A),
                                                  B.data_ptr(), Handle._ld(B), out.data_ptr(),
                                                  Handle._ld(out), ph)

@@ -79,7 +79,12 @@ CIGEMM_API cigemmStatus_t cigemm_probe_issue_cost(cigemmHandle_t handle, int n_d
  * acknowledged; microseconds from the first workgroup's start to the last one's end; shader
  * cycles per 64-byte stage of k in the main loop; shader clock (GHz) held in the main loop
  * (0 when the main loop is shorter than one tick of the wall clock); microseconds from the
- * first workgroup entering its epilogue to the last one's end; number of workgroups.
+ * first workgroup entering its epilogue to the last one's end; number of workgroups;
+ * phases[8..11]: main-loop shader clock (GHz) of the slowest and of the fastest of the chip's
+ * compute dies (XCDs: each holds its own clock, and every die gets the same number of
+ * workgroups); microseconds from the first workgroup's start to the end of a compute unit's last
+ * workgroup, averaged over the units (the launch itself, phases[3], ends with the slowest unit);
+ * number of compute units that ran a workgroup.  `phases` must hold 12 doubles.
  * Synchronises the stream; meant for profiling runs, not for the hot path. */
 CIGEMM_API cigemmStatus_t cigemm_probe_tile_phases(cigemmHandle_t handle, int kind, int64_t M,
                                                    int64_t N, int64_t K, const void* A,

@@ -47,6 +47,11 @@ def test_probe_output_equals_plain_call_and_phases_add_up(handle, torch_gpu, ora
         assert ph["prologue_us"] + ph["main_loop_us"] + ph["epilogue_us"] <= ph["first_start_to_last_end_us"] * 1.001
         assert ph["cycles_per_stage"] >= min_cycles
         assert 0.05 < ph["main_loop_clock_ghz"] < 3.0
+        # per die and per unit: the dies' clocks bracket the average, no unit ends after the launch
+        assert 0.05 < ph["slowest_xcd_clock_ghz"] <= ph["main_loop_clock_ghz"] * 1.001
+        assert ph["main_loop_clock_ghz"] <= ph["fastest_xcd_clock_ghz"] * 1.001 < 3.0
+        assert 1 <= ph["units"] <= min(tiles, 256)
+        assert 0 < ph["mean_unit_end_us"] <= ph["first_start_to_last_end_us"] * 1.001
 
 
 def test_probe_same_tile_mode(handle, torch_gpu, oracle, rng):
