@@ -48,3 +48,34 @@ def test_hot_kernels_do_not_spill():
             assert n <= 12, (name, n)      # (set-up values, spilled once outside the timed loop)
         else:
             assert n == 0, (name, n)
+
+
+@pytest.mark.skipif(HIPCC is None, reason="hipcc not installed")
+def test_cross_workgroup_exchange_uses_agent_scope_accesses():
+    """The decode kernels' K ranges meet through memory written by one workgroup and read by
+    another, possibly on another XCD whose L2 is not coherent with the writer's.  The code relies
+    on every such access being an agent-scope atomic, which gfx950 encodes as a load / store with
+    the sc1 bit (served at the memory-side point of coherence, never by the local L2), and on
+    there being NO whole-cache write-back or invalidate in those kernels (55 us per call).  A
+    compiler that stopped encoding either would break results only under particular timing; this
+    checks the generated code instead."""
+    with tempfile.TemporaryDirectory() as d:
+        out = os.path.join(d, "skinny.s")
+        subprocess.run([HIPCC, *FLAGS, os.path.join(CSRC, "gemm_skinny.hip"), "-o", out], check=True,
+                       stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        text = open(out).read()
+    kernels = re.split(r"\n(?=_Z\w+:)", text)
+    seen = 0
+    for body in kernels:
+        name = body.split(":", 1)[0]
+        if "skinny_kn16_kwaves_kernel" not in name and "skinny_kernelI" not in name:
+            continue
+        if re.search(r"skinny_kernelI.*ELi1EEEviii", name):
+            continue                       # one K range: nothing is exchanged
+        seen += 1
+        assert not re.search(r"\bbuffer_wbl2\b|\bbuffer_inv\b", body), name
+        # partial sums: 8-byte agent-scope stores and loads; the arrival counter: an atomic add
+        assert re.search(r"global_store_dwordx2 .* sc1", body), name
+        assert re.search(r"global_load_dwordx2 .* sc1", body), name
+        assert re.search(r"global_atomic_(add|swap)", body), name
+    assert seen >= 12
