@@ -300,6 +300,121 @@ def decode_sweep(torch, ci, handle, steps, warmup):
     print(json.dumps({"decode_sweep": res}), flush=True)
 
 
+PLAN_SWEEP_SHAPES = {
+    # (N, K) of the weights: layer shapes of common decoder models
+    "a": [(8192, 8192), (11008, 4096), (4096, 11008), (4096, 4096), (14336, 4096), (4096, 14336)],
+    "b": [(5120, 5120), (13824, 5120), (5120, 13824), (6144, 4096), (12288, 4096), (28672, 8192),
+          (8192, 28672), (10240, 8192), (2048, 2048), (3072, 8192), (8192, 3072), (7168, 7168),
+          (1024, 4096), (16384, 2048), (2048, 16384)],
+    "c": [(4096, 4096), (8192, 2048), (2048, 8192), (11008, 4096), (4096, 11008), (1024, 4096),
+          (5120, 5120)],
+    # not used when the planner's constants were chosen
+    "d": [(3584, 3584), (18944, 3584), (3584, 18944), (9216, 4608), (4608, 9216), (6656, 6656)],
+    "e": [(3584, 3584), (18944, 3584), (3584, 18944), (6656, 6656)],
+}
+PLAN_SWEEP_MS = {
+    "a": (33, 64, 65, 128, 129, 192, 256, 257, 384, 512, 768, 1024, 1536, 2048),
+    "b": (40, 72, 96, 128, 160, 200, 256, 320, 448, 512, 640, 896, 1024, 1280, 2048),
+    "c": (40, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 2048),
+    "d": (48, 100, 144, 224, 288, 352, 480, 576, 704, 960, 1152, 1792),
+    "e": (48, 100, 144, 224, 288, 352, 480, 576, 704, 960, 1152, 1792),
+}
+PLAN_SWEEP_KINDS = {"a": ("bf16", "i8nk"), "b": ("bf16", "i8nk"), "c": ("f32", "i8kn"),
+                    "d": ("bf16", "i8nk"), "e": ("f32", "i8kn")}
+
+
+def plan_sweep(torch, ci, probe, handle, sets, out_path):
+    """Evidence for the tile kernel's planner: for every problem of the chosen sets (batch sizes
+    between the decode kernels' and one full round of 256-row tiles) the library's own plan and
+    every imposed (tile rows, K ranges) plan are timed; prints, per problem, how much slower the
+    library's choice is than the best plan timed, and writes all timings as JSON."""
+    def timed(fn, steps, warm):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps * 1e3
+
+    out = []
+    for st in sets:
+        for kind in PLAN_SWEEP_KINDS[st]:
+            eb = {"bf16": 2, "f32": 4}.get(kind, 1)
+            for (N, K) in PLAN_SWEEP_SHAPES[st]:
+                nb = max(2, min(6, (600 << 20) // (K * N * eb)))   # rotated: no cache holds them
+                if kind == "bf16":
+                    ws = [(torch.randn((K, N), device="cuda") * 0.02).to(torch.bfloat16) for _ in range(nb)]
+                elif kind == "f32":
+                    ws = [torch.randn((K, N), device="cuda") * 0.02 for _ in range(nb)]
+                else:
+                    shape = (N, K) if kind == "i8nk" else (K, N)
+                    ws = [torch.randint(-127, 128, shape, dtype=torch.int8, device="cuda") for _ in range(nb)]
+                for M in PLAN_SWEEP_MS[st]:
+                    if kind == "bf16":
+                        x = torch.randn((M, K), device="cuda").to(torch.bfloat16)
+                        y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+                    elif kind == "f32":
+                        x = torch.randn((M, K), device="cuda")
+                        y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+                    else:
+                        x = torch.randint(-127, 128, (M, K), dtype=torch.int8, device="cuda")
+                        y = torch.empty((M, N), dtype=torch.int32, device="cuda")
+                    it = [0]
+
+                    def fn():
+                        w = ws[it[0] % nb]
+                        it[0] += 1
+                        if kind == "bf16":
+                            handle.gemm_bf16(x, w, out=y)
+                        elif kind == "f32":
+                            handle.gemm_f32(x, w, out=y)
+                        else:
+                            handle.gemm_i8_i32(x, w, ci.B_NK if kind == "i8nk" else ci.B_KN, out=y)
+                    probe.force_tile_plan(handle, 0)
+                    own = timed(fn, 60, 10)
+                    own_kernel, own_plan = handle.last_kernel, handle.last_plan
+                    plans = {}
+                    if own_plan[0]:     # the tile kernel serves this problem
+                        for rows in (64, 128, 192, 256):
+                            if rows > 64 and rows - 64 >= M:
+                                continue
+                            for sp in (1, 2, 3, 4, 5, 6, 7, 8, 10, 12, 16, 20, 24, 32):
+                                probe.force_tile_plan(handle, rows, sp)
+                                fn()
+                                torch.cuda.synchronize()
+                                pl = handle.last_plan
+                                key = f"{pl[0]}x{pl[1]}"
+                                tiles = -(-M // rows) * -(-N // 256) * pl[1]
+                                if key in plans or (tiles > 768 and pl[1] > 1):
+                                    continue
+                                plans[key] = round(timed(fn, 40, 10), 1)
+                        probe.force_tile_plan(handle, 0)
+                    rec = dict(kind=kind, M=M, N=N, K=K, own_us=round(own, 1), own_kernel=own_kernel,
+                               own_plan=list(own_plan), plans=plans)
+                    if plans:
+                        rec["best"] = min(plans, key=plans.get)
+                        rec["best_us"] = plans[rec["best"]]
+                        log(f"[plan-sweep] {kind} M={M} N={N} K={K}: own {own_plan[0]}x{own_plan[1]} "
+                            f"{own:.1f} us | best {rec['best']} {rec['best_us']:.1f} us | "
+                            f"{100 * (own / rec['best_us'] - 1):+.1f} %")
+                    out.append(rec)
+                del ws
+    losses = [r["own_us"] / r["best_us"] - 1 for r in out if r["plans"]]
+    summary = {"problems": len(losses), "mean_loss": sum(losses) / max(1, len(losses)),
+               "max_loss": max(losses, default=0.0),
+               "over_5_percent": sum(1 for v in losses if v > 0.05),
+               "over_10_percent": sum(1 for v in losses if v > 0.10)}
+    if out_path:
+        with open(out_path, "w") as f:
+            json.dump(out, f)
+    print(json.dumps({"plan_sweep": summary}), flush=True)
+
+
 ONLY_WORKLOADS = ("bf16_8192", "fp16_8192", "int8_8192", "int8_8192_nk", "int8_4096_dequant_f32",
                   "int8_linear_2048x11008x4096_dequant_bf16", "fp32_4096")
 
@@ -375,6 +490,11 @@ def main():
     ap.add_argument("--decode-sweep", action="store_true",
                     help="instead of the benchmark: decode GEMMs (M = 1, 16, 32) at layer shapes of common "
                          "decoder models, bf16 and int8")
+    ap.add_argument("--plan-sweep", metavar="SETS",
+                    help="instead of the benchmark: time every (tile rows, K ranges) plan of the tile "
+                         "kernel against the library's own choice over the problem sets named "
+                         "(letters of a..e; e.g. 'ab')")
+    ap.add_argument("--plan-sweep-out", default="", help="with --plan-sweep: write all timings here (JSON)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1",
@@ -395,6 +515,12 @@ def main():
         return
     if args.decode_sweep:
         decode_sweep(torch, ci, handle, args.steps, args.warmup)
+        return
+    if args.plan_sweep:
+        if any(c not in PLAN_SWEEP_SHAPES for c in args.plan_sweep):
+            print("--plan-sweep takes letters of: " + "".join(PLAN_SWEEP_SHAPES), file=sys.stderr)
+            sys.exit(2)
+        plan_sweep(torch, ci, probe, handle, args.plan_sweep, args.plan_sweep_out)
         return
     if args.only:
         only_workload(torch, ci, wl, handle, args.only, args.steps, args.warmup)

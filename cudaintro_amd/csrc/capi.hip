@@ -89,6 +89,8 @@ cigemmStatus_t cigemmCreate(cigemmHandle_t* handle) {
   ctx->ws_counter_bytes = (size_t)64 << 10;
   ctx->ws_swap_bytes = (size_t)8 << 20;  // 128 bytes per column: N <= 65536
   ctx->ws_dirty = 0;
+  ctx->force_tile_mt = 0;
+  ctx->force_tile_splits = 0;
   ctx->workspace = nullptr;
   if (hipMalloc(&ctx->workspace,
                 ctx->ws_partial_bytes + ctx->ws_counter_bytes + ctx->ws_swap_bytes) != hipSuccess ||

@@ -39,6 +39,11 @@ struct cigemmContext {
   // that did not run to its end may have left arrival counters or exchange words non-zero.
   // The next GEMM call clears both (a small kernel on the handle's stream) before it launches.
   int ws_dirty;
+  // Measurement aid, set through the probe library only: with force_tile_mt in 1..4 the tile
+  // kernel's launcher runs tiles of 64 * force_tile_mt rows over force_tile_splits K ranges
+  // in place of its own plan; 0 = the launcher chooses.
+  int force_tile_mt;
+  int force_tile_splits;
   char last_error[256];
 };
 

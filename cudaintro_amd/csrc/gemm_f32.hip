@@ -32,7 +32,8 @@ bool launch_f32_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const 
     const bool one_round = ((M + 255) / 256) * ((N + tile::BN - 1) / tile::BN) <= cus;
     const bool long_k_split =
         tile_ok && K >= 2048 && one_round &&
-        tile::plan_small(ctx, M, N, K * 4, tile::MathF32::STAGE_UNIT_US, K * 4 * N)
+        tile::plan_small(cus, ctx->workspace ? ctx->ws_partial_bytes : 0, M, N, K * 4, 4,
+                         tile::stage_cost<tile::MathF32, tile::B_KN32>(), K * 4 * N)
                 .splits > 1;
     // What the tile kernel cannot take (B or C rows not 16-byte aligned, an odd N) and fills the
     // chip with 128 x 128 tiles is left to the any-shape matrix-core kernel (4096 x 4095 x 4096:

@@ -61,12 +61,11 @@
 #include <type_traits>
 
 #include "common.h"
+#include "tile_plan.h"
 
 namespace cig {
 namespace tile {
 
-constexpr int BM = 256, BN = 256;
-constexpr int KB = 64;                     // bytes of k per stage, per row
 constexpr int OPERAND_BYTES = 256 * KB;    // 16 KiB, either operand
 
 typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
@@ -242,7 +241,6 @@ __device__ __forceinline__ typename BTile<MODE>::piece_t read_b_piece(const char
 // ---- arithmetic traits ----------------------------------------------------------------------
 struct MathBF16 {
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
-  static constexpr double STAGE_UNIT_US = 0.195;  // one 64 x 256 step of one 64-byte stage
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
   typedef f32x16 acc_t;
   typedef float scalar_t;
@@ -255,7 +253,6 @@ struct MathBF16 {
 };
 struct MathF16 {
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
-  static constexpr double STAGE_UNIT_US = 0.195;
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
   typedef f32x16 acc_t;
   typedef float scalar_t;
@@ -267,7 +264,6 @@ struct MathF16 {
 };
 struct MathI8 {
   static constexpr int SUBSTEPS = 1;  // MFMAs per fragment pair
-  static constexpr double STAGE_UNIT_US = 0.195;
   static __device__ __forceinline__ u32x4 afrag(u32x4 a, int) { return a; }
   typedef i32x16 acc_t;
   typedef int32_t scalar_t;
@@ -283,7 +279,6 @@ struct MathI8 {
 // so four MFMAs consume one fragment pair: MFMA e multiplies k0+e (lanes 0-31) and k0+4+e.
 struct MathF32 {
   static constexpr int SUBSTEPS = 4;
-  static constexpr double STAGE_UNIT_US = 0.95;
   static __device__ __forceinline__ float afrag(u32x4 a, int sub) {
     const uint32_t bits = a[sub];  // (bit_cast applied directly to a vector element misreads it)
     return __builtin_bit_cast(float, bits);
@@ -499,20 +494,26 @@ __device__ __forceinline__ void store_tile(const Epi& epi, typename Math::acc_t 
 // Epi: an epilogue functor (see epilogues.h): load_row / load_cols / pack / side / out_row.
 //
 // A, B are byte pointers; lda/ldb are in BYTES.  Any M; N a multiple of 4; all rows 16-byte
-// aligned (tile_shape_ok checks).  KTS = number of 64-byte stages of this workgroup's K
-// range, k_bytes = bytes of k in it (a multiple of 16; the last stage may be partly filled:
-// the pieces past k_bytes are fetched as zeros); grid = (tiles, K ranges).
+// aligned (tile_shape_ok checks).  grid = (tiles, K ranges): range y covers the bytes
+// [y * k_range_bytes, min((y + 1) * k_range_bytes, k_total_bytes)) of k; k_range_bytes is a
+// whole number of 64-byte stages whenever there is more than one range, so only the last
+// range can be shorter than the others or leave its last stage partly filled (the pieces
+// past its end are fetched as zeros).  k_total_bytes is a multiple of 16.
 template <typename Math, int BMODE, int NSTAGES, int MT, typename Epi, int WM = 2>
 __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, int tiles_m,
-                                                           int tiles_n, int KTS, int k_bytes,
+                                                           int tiles_n, int k_range_bytes,
+                                                           int k_total_bytes,
                                                            const char* __restrict__ A,
                                                            int64_t lda,
                                                            const char* __restrict__ B,
                                                            int64_t ldb, Epi epi_all,
                                                            int64_t a_split_step,
                                                            int64_t b_split_step) {
-  // blockIdx.y = K range (split-K launches only): KTS stages starting a_split_step /
-  // b_split_step bytes further per range
+  // blockIdx.y = K range (split-K launches only): each starts a_split_step / b_split_step
+  // bytes after the one before; k_bytes = bytes of k in this one, KTS = its stages
+  const int k_left = k_total_bytes - (int)blockIdx.y * k_range_bytes;
+  const int k_bytes = k_left < k_range_bytes ? k_left : k_range_bytes;
+  const int KTS = (k_bytes + KB - 1) / KB;
   const Epi epi = epilogue_of_split(epi_all, (int)blockIdx.y);
   A += blockIdx.y * a_split_step;
   B += blockIdx.y * b_split_step;
@@ -936,6 +937,7 @@ __global__ __launch_bounds__(128 * WM, 1) void mfma_tile_kernel(int M, int N, in
 
 constexpr int DEFAULT_STAGES = 4;
 
+// `splits` must be a value k_ranges() returned for this K (1 = the whole of K in one range).
 template <typename Math, int BMODE, int MT, typename Epi, int WM = 2>
 void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
                     int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi,
@@ -949,20 +951,20 @@ void launch_tile_mt(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, c
   static std::atomic<uint64_t> lds_set{0};  // one per template instance
   if (!ensure_dynamic_lds(ctx, (const void*)kern, LDS_BYTES, lds_set)) return;
   const int tiles_m = (int)((M + TILE_M - 1) / TILE_M), tiles_n = (int)((N + BN - 1) / BN);
+  int64_t range_stages = 0;
+  splits = k_ranges(K_bytes, splits, &range_stages);
   ctx->last_tile_rows = TILE_M;
   ctx->last_k_splits = splits;
   ctx->last_waves = 2 * WM;
   ctx->last_per_cu = 1;
-  // stages per K range; only an unsplit K may leave its last stage partly filled
-  const int64_t kts = splits > 1 ? K_bytes / KB / splits : (K_bytes + KB - 1) / KB;
-  const int64_t range_bytes = splits > 1 ? kts * KB : K_bytes;
-  const int64_t a_step = kts * KB;
-  const int64_t b_step = BMODE == B_NK ? kts * KB : kts * (KB / Math::ELEM_BYTES) * ldb_bytes;
+  const int64_t range_bytes = splits > 1 ? range_stages * KB : K_bytes;
+  const int64_t a_step = range_stages * KB;
+  const int64_t b_step =
+      BMODE == B_NK ? range_stages * KB : range_stages * (KB / Math::ELEM_BYTES) * ldb_bytes;
   hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(128 * WM),
-                     LDS_BYTES, ctx->stream, (int)M, (int)N, tiles_m, tiles_n, (int)kts,
-                     (int)range_bytes,
-                     static_cast<const char*>(A), lda_bytes, static_cast<const char*>(B),
-                     ldb_bytes, epi, a_step, b_step);
+                     LDS_BYTES, ctx->stream, (int)M, (int)N, tiles_m, tiles_n, (int)range_bytes,
+                     (int)K_bytes, static_cast<const char*>(A), lda_bytes,
+                     static_cast<const char*>(B), ldb_bytes, epi, a_step, b_step);
 }
 
 // Second half of a split-K GEMM: sums the `splits` partial matrices in split order (the
@@ -1006,77 +1008,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(int M, int N, int sp
   }
 }
 
-// Plan for a problem that fits one round of 256-row tiles: tile height and number of K
-// ranges, by estimated time.  Main launch: rounds x tile cost x stages per range, where short
-// tiles cost more per output than in the compute-bound plan below because such problems are
-// bound by the weight stream (bf16 512 x 8192 x 8192, 256 workgroups each: 256-row tiles and
-// 4 ranges 85 us, 128-row and 2 ranges 89 us, 64-row unsplit 102 us).  Split plans add the
-// reduction launch: a fixed 5 us plus (splits + 1) M N 4 bytes at 3 TB/s.  `sm_us` = time of
-// one 64 x 256 x (64-byte stage) step of the arithmetic type; `b_bytes` = size of B: when it
-// stays in the caches the compute-bound tile costs apply.
-struct SmallPlan {
-  int mt;
-  int splits;
-};
-// Cost of one tile of 64*mt rows, in units of a quarter of the 256-row tile's: a fixed part
-// (the B panel is fetched whatever the height) plus a part per 64 rows; the fixed part weighs
-// more when B streams from HBM than when it sits in the L2 / Infinity Cache.  One round of
-// 256 tiles, N = 4096, K = 1024..4096, 16-bit and int8: 4.0 / 3.1-3.2 / 2.3 / 1.6-1.8;
-// 2 x 32 tiles over 8192 x 8192 weights: 4.0 / 3.0-3.5 / 2.5 / 1.9-2.3.
-inline double tile_cost_units(int mt, bool streamed) {
-  return streamed ? 1.2 + 0.7 * mt : 0.8 + 0.8 * mt;
-}
-
-inline SmallPlan plan_small(const cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes,
-                            double sm_us, int64_t b_bytes) {
-  const int64_t kts = (K_bytes + KB - 1) / KB;
-  const bool whole_stages = K_bytes % KB == 0;  // K ranges are whole stages
-  const bool streamed = b_bytes > (16LL << 20);
-  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
-  SmallPlan best{0, 1};
-  double best_us = 1e30;
-  for (int mt : {4, 3, 2, 1}) {
-    if (mt > 1 && 64 * (mt - 1) >= M) continue;  // the next lower height already covers M
-    const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + BN - 1) / BN);
-    const double per_tile = tile_cost_units(mt, streamed);
-    for (int sp = 1; sp <= 16; sp *= 2) {
-      if (sp > 1) {
-        if (!ctx->workspace || !whole_stages || kts % sp || kts / sp < 8) break;
-        if ((size_t)sp * (size_t)M * (size_t)N * 4 > ctx->ws_partial_bytes) break;
-      }
-      // (every round also pays its ramp and its epilogue: about 4.5 us.  Without that term
-      // 11008 x 4096 at M <= 16 ran as 43 tiles x 16 ranges in three rounds, 27.9 us, where 4
-      // ranges in one round take 21.8.)
-      const double rounds = (double)((tiles * sp + cus - 1) / cus);
-      double us = rounds * (4.5 + per_tile * sm_us * (double)(kts / sp));
-      if (sp > 1) us += 5.0 + (double)(sp + 1) * (double)M * (double)N * 4.0 / 3.0e6;
-      if (us < best_us) {
-        best_us = us;
-        best = SmallPlan{mt, sp};
-      }
-    }
-  }
-  return best;
-}
-
-// Relative cost of covering M x N with tiles of 64*mt rows on `cus` compute units: rounds of
-// workgroups times the cost of one tile; shorter tiles re-read B more often per flop.
-inline double tile_plan_cost(int64_t M, int64_t N, int mt, int cus) {
-  const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + BN - 1) / BN);
-  return (double)((tiles + cus - 1) / cus) * tile_cost_units(mt, false);
-}
-inline int best_mt(int64_t M, int64_t N, int cus, double* cost = nullptr) {
-  int best = 0;
-  double bc = 1e30;
-  for (int mt : {4, 3, 2, 1}) {
-    const double c = tile_plan_cost(M, N, mt, cus);
-    if (c < bc) {
-      bc = c;
-      best = mt;
-    }
-  }
-  if (cost) *cost = bc;
-  return best;
+// What a stage costs a workgroup of each operand layout (see tile_plan.h).
+template <typename Math, int BMODE>
+constexpr StageCost stage_cost() {
+  if constexpr (BMODE == B_KN32) return STAGE_COST_KN32;
+  if constexpr (BMODE == B_KN16) return STAGE_COST_KN16;
+  if constexpr (BMODE == B_NK) return STAGE_COST_NK8;
+  return STAGE_COST_KN8;
 }
 
 // An epilogue may declare `static constexpr bool REGISTER_HEAVY = true` to stay on the
@@ -1136,6 +1074,31 @@ void launch_tile_any_mt(cigemmContext* ctx, int mt, int64_t M, int64_t N, int64_
     launch_tile_mt<Math, BMODE, 1>(ctx, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi, splits);
 }
 
+// Runs one plan: tiles of 64*mt rows; with more than one K range the ranges go over
+// blockIdx.y, partial sums to the workspace, then one reduction launch with the real epilogue.
+// Returns true when it ran as such a pair of launches.
+template <typename Math, int BMODE, typename Epi>
+bool run_tile_plan(cigemmContext* ctx, int mt, int splits, int64_t M, int64_t N, int64_t K_bytes,
+                   const void* A, int64_t lda_bytes, const void* B, int64_t ldb_bytes,
+                   const Epi& epi) {
+  if (splits <= 1) {
+    launch_tile_any_mt<Math, BMODE>(ctx, mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
+    return false;
+  }
+  typedef typename Math::scalar_t scalar_t;
+  const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  uint32_t* ws = static_cast<uint32_t*>(ctx->workspace);
+  const EpiPartialX4 part{ws, N, M * N};
+  launch_tile_any_mt<Math, BMODE>(ctx, mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, part,
+                                  splits);
+  const int64_t quads = M * (N / 4);
+  const unsigned grid = (unsigned)((quads + 255) / 256 < 4 * (int64_t)cus ? (quads + 255) / 256
+                                                                          : 4 * (int64_t)cus);
+  hipLaunchKernelGGL((splitk_reduce_kernel<scalar_t, Epi>), dim3(grid), dim3(256), 0, ctx->stream,
+                     (int)M, (int)N, ctx->last_k_splits, ws, M * N, epi);
+  return true;
+}
+
 // Chooses the tile height, and, when the last round of 256-row tiles would leave most of the
 // chip idle, covers the columns of the full rounds with 256-row tiles and the remaining
 // columns with a second launch of shorter tiles.  Epi::shift_cols(c) returns the epilogue of
@@ -1145,29 +1108,27 @@ template <typename Math, int BMODE, typename Epi>
 bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, const void* A,
                  int64_t lda_bytes, const void* B, int64_t ldb_bytes, const Epi& epi) {
   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  if (ctx->force_tile_mt >= 1 && ctx->force_tile_mt <= 4) {
+    // a plan imposed through the measurement library: as asked, but for K ranges the
+    // workspace cannot hold
+    int64_t range_stages = 0;
+    int sp = k_ranges(K_bytes, ctx->force_tile_splits, &range_stages);
+    if (sp > 1 && (!ctx->workspace ||
+                   (size_t)sp * (size_t)M * (size_t)N * 4 > ctx->ws_partial_bytes))
+      sp = 1;
+    return run_tile_plan<Math, BMODE>(ctx, ctx->force_tile_mt, sp, M, N, K_bytes, A, lda_bytes, B,
+                                      ldb_bytes, epi);
+  }
   double single = 0;
   const int mt = best_mt(M, N, cus, &single);
   if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) <= cus) {
     // At most one round of 256-row tiles: pick the tile height and the number of K ranges
-    // together.  Split plans run K over blockIdx.y, partial sums to the workspace, then one
-    // reduction launch with the real epilogue.
-    const SmallPlan plan = plan_small(ctx, M, N, K_bytes, Math::STAGE_UNIT_US, K_bytes * N);
-    if (plan.splits > 1) {
-      typedef typename Math::scalar_t scalar_t;
-      uint32_t* ws = static_cast<uint32_t*>(ctx->workspace);
-      const EpiPartialX4 part{ws, N, M * N};
-      launch_tile_any_mt<Math, BMODE>(ctx, plan.mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes,
-                                      part, plan.splits);
-      const int64_t quads = M * (N / 4);
-      const unsigned grid = (unsigned)((quads + 255) / 256 < 4 * (int64_t)cus
-                                           ? (quads + 255) / 256
-                                           : 4 * (int64_t)cus);
-      hipLaunchKernelGGL((splitk_reduce_kernel<scalar_t, Epi>), dim3(grid), dim3(256), 0,
-                         ctx->stream, (int)M, (int)N, plan.splits, ws, M * N, epi);
-      return true;
-    }
-    launch_tile_any_mt<Math, BMODE>(ctx, plan.mt, M, N, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
-    return false;
+    // together.
+    const SmallPlan plan =
+        plan_small(cus, ctx->workspace ? ctx->ws_partial_bytes : 0, M, N, K_bytes, Epi::OUT_BYTES,
+                   stage_cost<Math, BMODE>(), K_bytes * N);
+    return run_tile_plan<Math, BMODE>(ctx, plan.mt, plan.splits, M, N, K_bytes, A, lda_bytes, B,
+                                      ldb_bytes, epi);
   }
   {
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;

@@ -457,3 +457,19 @@ extern "C" cigemmStatus_t cigemm_probe_dirty_workspace(cigemmHandle_t h, int cou
   if (mark_dirty) h->ws_dirty = 1;
   return CIGEMM_STATUS_SUCCESS;
 }
+
+extern "C" cigemmStatus_t cigemm_probe_force_tile_plan(cigemmHandle_t h, int tile_rows,
+                                                       int k_ranges) {
+  const char* name = "cigemm_probe_force_tile_plan";
+  if (!h || h->magic != kCtxMagic) return CIGEMM_STATUS_NOT_INITIALIZED;
+  if (tile_rows == 0) {
+    h->force_tile_mt = h->force_tile_splits = 0;
+    return CIGEMM_STATUS_SUCCESS;
+  }
+  if (tile_rows % 64 || tile_rows < 64 || tile_rows > 256 || k_ranges < 1 || k_ranges > 64)
+    return fail(h, CIGEMM_STATUS_INVALID_VALUE, "%s: tile_rows %d, k_ranges %d", name, tile_rows,
+                k_ranges);
+  h->force_tile_mt = tile_rows / 64;
+  h->force_tile_splits = k_ranges;
+  return CIGEMM_STATUS_SUCCESS;
+}

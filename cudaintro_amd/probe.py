@@ -29,6 +29,7 @@ SIGNATURES = {
     "cigemm_probe_gemm_i8_dequant_paired": (_ci, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _ci,
                                                   _vp, _ci, _vp, _ci, _i64, _vp, _i64]),
     "cigemm_probe_dirty_workspace": (_ci, [_vp, _ci, C.c_uint32, _ci]),
+    "cigemm_probe_force_tile_plan": (_ci, [_vp, _ci, _ci]),
 }
 
 
@@ -156,3 +157,10 @@ def gemm_i8_dequant_paired(h: Handle, A, B, scale_a, scale_b, out_type=OUT_F32, 
 def dirty_workspace(h: Handle, count: int, value: int, mark_dirty: bool):
     _check(h, load_library().cigemm_probe_dirty_workspace(h.raw, count, value, int(mark_dirty)),
            "cigemm_probe_dirty_workspace")
+
+
+def force_tile_plan(h: Handle, tile_rows: int, k_ranges: int = 1):
+    """Imposes the tile kernel's plan on the handle's following calls; tile_rows = 0 hands the
+    choice back to the library."""
+    _check(h, load_library().cigemm_probe_force_tile_plan(h.raw, tile_rows, k_ranges),
+           "cigemm_probe_force_tile_plan")

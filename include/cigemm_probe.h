@@ -124,6 +124,15 @@ CIGEMM_API cigemmStatus_t cigemm_probe_gemm_i8_dequant_paired(
 CIGEMM_API cigemmStatus_t cigemm_probe_dirty_workspace(cigemmHandle_t handle, int count,
                                                        uint32_t value, int mark_dirty);
 
+/* Planner evidence: imposes the tile kernel's plan on the handle's following GEMM calls (those
+ * the tile kernel serves): output tiles of `tile_rows` rows (64, 128, 192 or 256) over
+ * `k_ranges` ranges of K (1 = unsplit; rounded to ranges of an even number of 64-byte stages;
+ * run unsplit when the handle's workspace cannot hold the partial sums).  tile_rows = 0 hands
+ * the choice back to the library.  cigemmGetLastPlan() reports what ran.  Results are those of
+ * the library's own plan up to the order of the K ranges' floating-point sum. */
+CIGEMM_API cigemmStatus_t cigemm_probe_force_tile_plan(cigemmHandle_t handle, int tile_rows,
+                                                       int k_ranges);
+
 #ifdef __cplusplus
 }
 #endif

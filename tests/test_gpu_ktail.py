@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 import cudaintro_amd as ci
+from cudaintro_amd import probe
 from gpu_util import bits, error_bound_16
 
 pytestmark = pytest.mark.gpu
@@ -53,7 +54,7 @@ def test_k_tail_16bit(handle, torch_gpu, oracle, rng, kind, M, N, K):
     out = torch.full((M + 1, N + 8), 3.0, dtype=a.dtype, device="cuda")
     with handle.algo(ci.ALGO_TILE):
         fn(a, b, out=out[:M, :N])
-    assert handle.last_plan[1] == 1
+    assert handle.last_plan[0] > 0      # (a long K may run as several K ranges: the last holds the tail)
     o = bits(torch, out)
     if exact:
         np.testing.assert_array_equal(o[:M, :N], narrow(oracle.gemm_f32(widen(Ab), widen(Bb))))
@@ -154,3 +155,48 @@ def test_tail_shapes_keep_the_tile_kernel_by_default(handle, torch_gpu):
     b8 = torch.zeros((1008, 512), dtype=torch.int8, device="cuda")
     handle.gemm_i8_i32(a8, b8, ci.B_KN)
     assert "_mfma_" in handle.last_kernel, handle.last_kernel
+
+
+@pytest.mark.parametrize("rows,ranges", [(64, 2), (128, 3), (192, 5), (256, 7), (128, 16)])
+@pytest.mark.parametrize("K", [1000, 2048 + 16, 4096 + 24, 4096 - 40])
+def test_k_tail_in_the_last_k_range(handle, torch_gpu, oracle, rng, rows, ranges, K):
+    """Split plans imposed on a K with a tail: ranges of an even number of whole stages, the last
+    one shorter and ending in a partly filled stage.  Exact inputs: bit-equal to the CPU loop for
+    bf16 (K x N), int8 (both layouts) and fp32."""
+    torch = torch_gpu
+    M, N = 200, 528
+    try:
+        probe.force_tile_plan(handle, rows, ranges)
+        # bf16
+        Af, Bf = rng.choice(VALS, size=(M, K)), rng.choice(VALS, size=(K, N))
+        Ab, Bb = oracle.f32_to_bf16(Af), oracle.f32_to_bf16(Bf)
+        a, b = dev16_padded(torch, Ab, "bf16", 1, 24), dev16_padded(torch, Bb, "bf16", 3, 8)
+        out = torch.full((M + 1, N + 8), 3.0, dtype=a.dtype, device="cuda")
+        with handle.algo(ci.ALGO_TILE):
+            handle.gemm_bf16(a, b, out=out[:M, :N])
+        got_rows, got_ranges = handle.last_plan
+        assert got_rows == rows and 1 < got_ranges <= ranges, handle.last_plan
+        np.testing.assert_array_equal(bits(torch, out)[:M, :N], oracle.f32_to_bf16(
+            oracle.gemm_f32(oracle.bf16_to_f32(Ab), oracle.bf16_to_f32(Bb))))
+        # fp32 (K in floats: the same byte counts at a quarter of the elements)
+        Kf = K // 2
+        Af, Bf = rng.choice(VALS, size=(M, Kf)), rng.choice(VALS, size=(Kf, N))
+        a, b = padded(torch, Af, torch.float32, 1, 12, float("nan")), padded(torch, Bf, torch.float32, 3, 8, float("nan"))
+        with handle.algo(ci.ALGO_TILE):
+            c = handle.gemm_f32(a, b)
+        assert handle.last_plan[0] == rows and handle.last_plan[1] > 1, handle.last_plan
+        np.testing.assert_array_equal(c.cpu().numpy(), oracle.gemm_f32(Af, Bf))
+        # int8, both layouts
+        for layout in (ci.B_KN, ci.B_NK):
+            nk = layout == ci.B_NK
+            K8 = 2 * K
+            A = rng.integers(-127, 128, size=(M, K8), dtype=np.int8)
+            B = rng.integers(-127, 128, size=(N, K8) if nk else (K8, N), dtype=np.int8)
+            a = padded(torch, A, torch.int8, 1, 48, 127)
+            b = padded(torch, B, torch.int8, 1, 48, 127) if nk else padded(torch, B, torch.int8, 5, 16, 127)
+            with handle.algo(ci.ALGO_TILE):
+                y = handle.gemm_i8_i32(a, b, layout)
+            assert handle.last_plan[0] == rows and handle.last_plan[1] > 1, handle.last_plan
+            np.testing.assert_array_equal(y.cpu().numpy(), oracle.gemm_i8_i32(A, B, b_is_nk=nk))
+    finally:
+        probe.force_tile_plan(handle, 0)

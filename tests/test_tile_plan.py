@@ -1,0 +1,48 @@
+"""The tile kernel's launch planning (csrc/tile_plan.h), on the host: invariants of the K ranges
+and of the chosen plans, and how the choice ranks against plans timed on an MI355X."""
+import json
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def planner(tmp_path_factory):
+    exe = tmp_path_factory.mktemp("tile_plan") / "test_tile_plan"
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-Werror", "-I", os.path.join(ROOT, "cudaintro_amd", "csrc"),
+                    os.path.join(ROOT, "tests", "cpp", "test_tile_plan.cpp"), "-o", str(exe)], check=True)
+    return str(exe)
+
+
+def test_tile_plan_invariants(planner):
+    out = subprocess.run([planner], capture_output=True, text=True)
+    assert out.returncode == 0 and "tile plan OK" in out.stdout, out.stdout[-2000:]
+
+
+def test_tile_plan_ranks_well_against_timed_plans(planner):
+    """tests/golden/tile_plan_sweep.json holds, for 253 problems (batch sizes 33..2048 over weight
+    shapes of common decoder layers; bf16, int8 in both layouts, fp32), the time of every
+    (tile rows, K ranges) plan, measured on an MI355X (bench.py --plan-sweep).  The planner's
+    choice must stay close to the best plan timed: 2 % slower on average when this was written
+    (the rule it replaced: 4.3 %, one problem in six more than 10 % slower)."""
+    with open(os.path.join(ROOT, "tests", "golden", "tile_plan_sweep.json")) as f:
+        problems = json.load(f)
+    lines = "".join(f"{p['kind']} {p['M']} {p['N']} {p['K']}\n" for p in problems)
+    out = subprocess.run([planner, "plan"], input=lines, capture_output=True, text=True, check=True)
+    picks = [tuple(map(int, ln.split())) for ln in out.stdout.split("\n") if ln.strip()]
+    assert len(picks) == len(problems)
+    losses = []
+    for p, (rows, sp) in zip(problems, picks):
+        key = f"{rows}x{sp}"
+        if key not in p["plans"]:
+            continue     # a plan the sweep did not time (more K ranges than it tried)
+        losses.append(p["plans"][key] / min(p["plans"].values()) - 1)
+    assert len(losses) >= 0.9 * len(problems), (len(losses), len(problems))
+    mean = sum(losses) / len(losses)
+    over10 = sum(1 for v in losses if v > 0.10) / len(losses)
+    assert mean < 0.03, mean
+    assert over10 < 0.06, over10
+    assert max(losses) < 0.40, max(losses)
