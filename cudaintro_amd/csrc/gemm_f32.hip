@@ -27,14 +27,11 @@ bool launch_f32_mfma(cigemmContext* ctx, int64_t M, int64_t N, int64_t K, const 
     tile::best_mt(M, N, cus, &tile_cost);
     const double tiles32 = (double)((M + 31) / 32) * (double)((N + 31) / 32);
     const double small_cost = 0.115 * (tiles32 > cus ? tiles32 / cus : 1.0);
-    // With a long K the tile kernel splits K over the idle compute units and wins
-    // (512 x 512 x 4096: 33 us against 55 us; 1024^3: 31 against 32; 512^3: 17 against 9).
+    // With a long K the tile kernel wins whenever its tiles fit one round: it can split K over
+    // the idle compute units (512 x 512 x 4096: 33 us against 55 us; 1024^3: 31 against 32;
+    // 512^3: 17 against 9; 960 x 3584 x 3584: 222 against 298).
     const bool one_round = ((M + 255) / 256) * ((N + tile::BN - 1) / tile::BN) <= cus;
-    const bool long_k_split =
-        tile_ok && K >= 2048 && one_round &&
-        tile::plan_small(cus, ctx->workspace ? ctx->ws_partial_bytes : 0, M, N, K * 4, 4,
-                         tile::stage_cost<tile::MathF32, tile::B_KN32>(), K * 4 * N)
-                .splits > 1;
+    const bool long_k_split = tile_ok && K >= 2048 && one_round;
     // What the tile kernel cannot take (B or C rows not 16-byte aligned, an odd N) and fills the
     // chip with 128 x 128 tiles is left to the any-shape matrix-core kernel (4096 x 4095 x 4096:
     // 109 against 63 TFLOP/s; at 1000^3, 64 such tiles, this kernel is 3x the faster one).

@@ -29,21 +29,24 @@ inline int k_ranges(int64_t K_bytes, int wanted, int64_t* range_stages) {
 }
 
 // Plan for a problem that fits one round of 256-row tiles: tile height and number of K
-// ranges, by estimated time.  The estimate has the terms that decide between such plans, with
-// constants chosen so that it ranks the plans of a measured sweep well (759 problems: M 33..2048
-// over weight shapes of common decoder layers, every tile height x 1..16 ranges timed; the plan
-// it picks is on average 2 % slower than the best one timed, see the header comment of
-// PlanCost), not so that each term is a calibrated time:
-//   one round of workgroups = a fixed cost + stages per range x cost of a stage + this round's
-//   share of the bytes that have to come from HBM (both operands once, plus the partial sums or
-//   the output, weighted) at a streaming rate; a last, partly filled round is priced by its own
-//   number of workgroups;
-//   a split plan adds the reduction launch as measured: max(4.75, 1.1 + bytes / 5.3 TB/s) us
+// ranges, by estimated time.  The estimate has the terms that decide between such plans; its
+// constants were chosen so that it ranks the plans of a timed sweep well (759 problems: batch
+// sizes 33..2048 over weight shapes of common decoder layers, bf16, int8 in both layouts and
+// fp32, every tile height x 1..32 ranges timed; tests/test_tile_plan.py checks the ranking
+// against those timings) and, second, so that it stays near the times themselves (rms error 12 %
+// on plans within 30 % of the best).  The plan it picks is 2 % slower than the best plan timed
+// on average, on those problems and on 237 others first timed afterwards.
+//   One round of workgroups = a fixed cost + stages per range x cost of a stage + this round's
+//   share of the memory traffic (both operands once, plus the partial sums or the output,
+//   weighted) at a streaming rate; a last, partly filled round is priced by its own number of
+//   workgroups.
+//   A split plan adds the reduction launch as measured: max(4.75, 1.1 + bytes / 5.3 TB/s) us
 //   for `splits` fp32 partial matrices read and one output written.
 // A stage costs a workgroup a part that does not depend on the tile height (it waits for its
 // operands: with three stages in flight the wait per stage is a third of the memory latency,
 // less when B sits in the L2 / Infinity Cache) plus a part per 64 rows (LDS reads and matrix
-// instructions).
+// instructions; fp32, whose matrix instructions are 16 times slower, is the one layout where
+// that part dominates).
 struct SmallPlan {
   int mt;
   int splits;
@@ -58,6 +61,8 @@ constexpr StageCost STAGE_COST_NK8{0.327, 0.008};
 constexpr StageCost STAGE_COST_KN8{0.261, 0.037};
 constexpr StageCost STAGE_COST_KN32{0.061, 0.746};
 struct PlanCost {
+  // (the fixed cost of a round came out near zero: what a launch costs whatever the plan does
+  // not help to choose one)
   static constexpr double ROUND_US = 0.05;         // ramp and epilogue of a round of workgroups
   static constexpr double LATER_ROUND_US = 0.05;   // the same for a partly filled last round
   static constexpr double HBM_TB_S = 9.0;
