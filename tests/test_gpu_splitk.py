@@ -158,3 +158,35 @@ def test_handle_recovers_after_a_failed_launch(torch_gpu, oracle, rng):
         probe.dirty_workspace(h, 8192, 7, mark_dirty=True)
         assert all(torch.equal(a, b) for a, b in zip(run_all(), want))
         assert all(torch.equal(a, b) for a, b in zip(run_all(), want))
+
+
+def test_full_rounds_then_a_planned_remainder(handle, torch_gpu, oracle, rng):
+    """Several rounds of tiles whose row tiles do not divide the unit count (6 x 43 tiles of 256
+    rows): the columns of the full rounds run as 256-row tiles, the last tile column as a second
+    launch of 64-row tiles over K ranges with its own reduction.  Exact-arithmetic inputs: bit
+    for bit the CPU loop, for bf16 and for int8 with per-row x per-column scales (whose column
+    scales must move with the column offset of the second launch)."""
+    torch = torch_gpu
+    if torch.cuda.get_device_properties(0).multi_processor_count != 256:
+        pytest.skip("the expected plan is that of a 256-CU device")
+    M, N, K = 1536, 11008, 1024
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    A, B = rng.choice(vals, size=(M, K)), rng.choice(vals, size=(K, N))
+    out = handle.gemm_bf16(to_dev(torch, oracle.f32_to_bf16(A), "bf16"), to_dev(torch, oracle.f32_to_bf16(B), "bf16"))
+    assert re.fullmatch(r"bf16_mfma_256\+\d+x256x32_w4\+w\d_ring4(_splitk)?", handle.last_kernel), handle.last_kernel
+    np.testing.assert_array_equal(bits(torch, out), oracle.f32_to_bf16(oracle.gemm_f32(A, B)))
+    K8 = 4096
+    A8 = rng.integers(-127, 128, size=(M, K8), dtype=np.int8)
+    for nk in (False, True):
+        B8 = rng.integers(-127, 128, size=(N, K8) if nk else (K8, N), dtype=np.int8)
+        sa = rng.uniform(1e-3, 5e-2, M).astype(np.float32)
+        sb = rng.uniform(1e-3, 5e-2, N).astype(np.float32)
+        layout = ci.B_NK if nk else ci.B_KN
+        y = handle.gemm_i8_dequant(torch.from_numpy(A8).cuda(), torch.from_numpy(B8).cuda(),
+                                   torch.from_numpy(sa).cuda(), torch.from_numpy(sb).cuda(), layout, ci.OUT_BF16)
+        assert re.fullmatch(r"i8_mfma_256\+\d+x256x64_w\d\+w\d_ring4_(kn|nk)_dequant(_splitk)?", handle.last_kernel), \
+            handle.last_kernel
+        assert handle.last_kernel.endswith("_splitk"), handle.last_kernel
+        acc = oracle.gemm_i8_i32(A8, B8, b_is_nk=nk)
+        expect = oracle.dequant(acc, sa, sb, out_dtype="bf16", sa_per_row=True, sb_per_col=True)
+        np.testing.assert_array_equal(bits(torch, y), expect)
