@@ -1120,7 +1120,8 @@ bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
                                       ldb_bytes, epi);
   }
   double single = 0;
-  const int mt = best_mt(M, N, cus, &single);
+  constexpr TileUnits units = BMODE == B_KN32 ? TILE_UNITS_F32 : TILE_UNITS;
+  const int mt = best_mt(M, N, cus, &single, units);
   if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) <= cus) {
     // At most one round of 256-row tiles: pick the tile height and the number of K ranges
     // together.
@@ -1145,11 +1146,11 @@ bool launch_tile(cigemmContext* ctx, int64_t M, int64_t N, int64_t K_bytes, cons
       if (full_cols > 0 && full_cols < tiles_n) {
         const int64_t n1 = full_cols * BN, n2 = N - n1;
         double rest = 0;
-        const int mt2 = best_mt(M, n2, cus, &rest);
+        const int mt2 = best_mt(M, n2, cus, &rest, units);
         // (a tie stays with the single launch: int8 2048 x 11008 x 4096, 473 tiles of 192 rows in
         // two rounds against 256 tiles of 256 rows + 176 of 128 rows, alternating in one process:
         // 85.3 against 86.0 us)
-        if (tile_plan_cost(M, n1, 4, cus) + rest < single * 0.97) {
+        if (tile_plan_cost(M, n1, 4, cus, units) + rest < single * 0.97) {
           launch_tile_256<Math, BMODE>(ctx, M, n1, K_bytes, A, lda_bytes, B, ldb_bytes, epi);
           const int rows1 = ctx->last_tile_rows, waves1 = ctx->last_waves;
           const char* B2 = static_cast<const char*>(B) +

@@ -132,20 +132,31 @@ inline SmallPlan plan_small(int cus, size_t partial_bytes, int64_t M, int64_t N,
 // Cost of one tile of 64*mt rows in a plan of several rounds (compute bound), in units of a
 // quarter of the 256-row tile's: a fixed part (the B panel is fetched whatever the height) plus
 // a part per 64 rows.  One round of 256 tiles, N = 4096, K = 1024..4096, 16-bit and int8:
-// 4.0 / 3.1-3.2 / 2.3 / 1.6-1.8.
-inline double tile_cost_units(int mt) { return 0.8 + 0.8 * mt; }
+// 4.0 / 3.1-3.2 / 2.3 / 1.6-1.8.  fp32, whose matrix instructions are 16 times slower, pays
+// almost by the row (TILE_UNITS_F32): 5120 x 4096 x 4096 on 64-row tiles 1179 us against 1362 on
+// 192-row ones, 7000 x 4096 x 11008 4481 against 4875 on 256-row ones, 8192 x 6144 x 4096 2808
+// against 2733 (there the rounds fit).
+struct TileUnits {
+  double fixed, per_64_rows;
+};
+constexpr TileUnits TILE_UNITS{0.8, 0.8};
+constexpr TileUnits TILE_UNITS_F32{0.1, 0.975};
+inline double tile_cost_units(int mt, TileUnits u = TILE_UNITS) {
+  return u.fixed + u.per_64_rows * mt;
+}
 
 // Relative cost of covering M x N with tiles of 64*mt rows on `cus` compute units: rounds of
 // workgroups times the cost of one tile; shorter tiles re-read B more often per flop.
-inline double tile_plan_cost(int64_t M, int64_t N, int mt, int cus) {
+inline double tile_plan_cost(int64_t M, int64_t N, int mt, int cus, TileUnits u = TILE_UNITS) {
   const int64_t tiles = ((M + 64 * mt - 1) / (64 * mt)) * ((N + BN - 1) / BN);
-  return (double)((tiles + cus - 1) / cus) * tile_cost_units(mt);
+  return (double)((tiles + cus - 1) / cus) * tile_cost_units(mt, u);
 }
-inline int best_mt(int64_t M, int64_t N, int cus, double* cost = nullptr) {
+inline int best_mt(int64_t M, int64_t N, int cus, double* cost = nullptr,
+                   TileUnits u = TILE_UNITS) {
   int best = 0;
   double bc = 1e30;
   for (int mt : {4, 3, 2, 1}) {
-    const double c = tile_plan_cost(M, N, mt, cus);
+    const double c = tile_plan_cost(M, N, mt, cus, u);
     if (c < bc) {
       bc = c;
       best = mt;

@@ -84,6 +84,10 @@ static void check_plans() {
   // tile heights of plans of several rounds
   CHECK(best_mt(8192, 8192, 256) == 4, "8192^2: %d", best_mt(8192, 8192, 256));
   CHECK(best_mt(2048, 11008, 256) == 3, "2048 x 11008: %d", best_mt(2048, 11008, 256));
+  // fp32 pays by the row: short tiles where they waste fewer rounds
+  CHECK(best_mt(5120, 4096, 256, nullptr, TILE_UNITS_F32) == 1, "fp32 5120 x 4096");
+  CHECK(best_mt(8192, 6144, 256, nullptr, TILE_UNITS_F32) == 4, "fp32 8192 x 6144");
+  CHECK(best_mt(4096, 4096, 256, nullptr, TILE_UNITS_F32) == 4, "fp32 4096 x 4096");
 }
 
 int main(int argc, char** argv) {
