@@ -178,6 +178,61 @@ def test_random_int8(handle, torch_gpu, oracle, layout, case):
             np.testing.assert_array_equal(got, expect, err_msg=handle.last_kernel)
 
 
+SPLIT_PLANS = set()   # (tile rows, K ranges) the long-K cases below ran as
+
+
+def long_k_cases(seed, n):
+    """Batch sizes between the decode kernels' and a full round of tiles, with a K long enough
+    for the tile kernel to cut it into ranges: any count of ranges, the last one shorter, and a
+    K that ends inside a 64-byte stage."""
+    r = np.random.Generator(np.random.PCG64(seed))
+    out = []
+    for _ in range(n):
+        M = int(r.integers(33, 420))
+        N = int(r.integers(2, 80)) * 16
+        K = int(r.integers(64, 560)) * 16 + int(r.choice([0, 0, 16, 32, 48]))
+        out.append((M, N, K))
+    return out
+
+
+@pytest.mark.parametrize("case", long_k_cases(404, 36), ids=lambda c: f"{c[0]}x{c[1]}x{c[2]}")
+def test_random_long_k_split_plans(handle, torch_gpu, oracle, case):
+    """Exact-arithmetic inputs: bit for bit the CPU loop whatever plan the library takes, for
+    bf16, fp32 (a quarter of the k) and int8 in both layouts."""
+    torch = torch_gpu
+    M, N, K = case
+    r = np.random.Generator(np.random.PCG64(M * 1000003 + N * 1009 + K))
+    vals = np.array([0, 0.5, -0.5, 1, -1, 2, -2], np.float32)
+    A, B = r.choice(vals, size=(M, K)), r.choice(vals, size=(K, N))
+    out = handle.gemm_bf16(to_dev(torch, oracle.f32_to_bf16(A), "bf16"), to_dev(torch, oracle.f32_to_bf16(B), "bf16"))
+    SPLIT_PLANS.add(handle.last_plan)
+    np.testing.assert_array_equal(bits(torch, out), oracle.f32_to_bf16(oracle.gemm_f32(A, B)),
+                                  err_msg=f"{handle.last_kernel} {handle.last_plan}")
+    Kf = K // 4 * 4 // 2
+    Kf -= Kf % 4
+    Af, Bf = r.choice(vals, size=(M, Kf)), r.choice(vals, size=(Kf, N))
+    c = handle.gemm_f32(torch.from_numpy(Af).cuda(), torch.from_numpy(Bf).cuda())
+    SPLIT_PLANS.add(handle.last_plan)
+    np.testing.assert_array_equal(c.cpu().numpy(), oracle.gemm_f32(Af, Bf),
+                                  err_msg=f"{handle.last_kernel} {handle.last_plan}")
+    A8 = r.integers(-127, 128, size=(M, K), dtype=np.int8)
+    for nk in (False, True):
+        B8 = r.integers(-127, 128, size=(N, K) if nk else (K, N), dtype=np.int8)
+        y = handle.gemm_i8_i32(torch.from_numpy(A8).cuda(), torch.from_numpy(B8).cuda(), ci.B_NK if nk else ci.B_KN)
+        SPLIT_PLANS.add(handle.last_plan)
+        np.testing.assert_array_equal(y.cpu().numpy(), oracle.gemm_i8_i32(A8, B8, b_is_nk=nk),
+                                      err_msg=f"{handle.last_kernel} {handle.last_plan}")
+
+
+def test_random_long_k_cases_reach_uneven_splits():
+    """... and only if the library did cut K: several different counts of ranges, odd ones too,
+    on several tile heights."""
+    ranges = {p[1] for p in SPLIT_PLANS if p[0] > 0}
+    rows = {p[0] for p in SPLIT_PLANS if p[1] > 1}
+    assert len(ranges) >= 6 and any(s > 1 and s % 2 for s in ranges), sorted(SPLIT_PLANS)
+    assert len(rows) >= 2, sorted(SPLIT_PLANS)
+
+
 def test_random_cases_reach_every_family():
     """The draws above are only worth something if they exercise the fast paths too."""
     for frag in ("f32_generic", "f32_mfma_small", "x256x16_w", "bf16_generic", "bf16_mfma_",
