@@ -23,6 +23,8 @@ PROGRAMS = {
                             "-I", "/opt/rocm/include"], "test_host_protocol.cpp", [], "host protocol OK"),
     "test_skinny_plan": (["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(ROOT, "cudaintro_amd", "csrc")],
                          "test_skinny_plan.cpp", [], "skinny plan OK"),
+    "test_tile_plan": (["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(ROOT, "cudaintro_amd", "csrc")],
+                       "test_tile_plan.cpp", [], "tile plan OK"),
     # (the sweep over all 2^24 numerators runs some ten times slower instrumented: still seconds)
     "test_exact_arith": (["gcc", "-O2", "-std=c11", "-ffp-contract=off", "-Wall"], "test_exact_arith.c", ["-lm"],
                          "exact arithmetic OK"),
