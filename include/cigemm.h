@@ -123,7 +123,8 @@ CIGEMM_API int cigemmGetVersion(void);
  * profiles).  The LDS-tiled matrix-core kernel reports its real plan:
  * "<type>_mfma_<tile rows>x256x<k per stage>_w<waves per workgroup>_ring4[_kn|_nk][_dequant]
  * [_bias_act][_splitk]", e.g. "bf16_mfma_256x256x32_w4_ring4", "i8_mfma_256+192x256x64_w8+w4_
- * ring4_nk_dequant" when two launches of different tile heights covered the columns.  Valid
+ * ring4_nk_dequant" when two launches of different tile heights covered the columns (a
+ * "_splitk" after such a name: the second launch ran as K ranges plus a reduction).  Valid
  * until the next GEMM call on the handle. */
 CIGEMM_API const char* cigemmGetLastKernelName(cigemmHandle_t handle);
 
